@@ -1,0 +1,135 @@
+"""ctypes binding of libf3s_amd.so (include/f3s_amd.h), operating on torch device tensors.
+
+This is the thinnest possible host layer: it passes data_ptr()s and sizes through the C ABI
+and raises RuntimeError with f3s_last_error() on a non-zero status. There is no fallback: if
+the HIP library is missing, importing or calling anything here fails.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libf3s_amd.so")
+_lib = None
+
+EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
+           "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd"]
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libf3s_amd.so is not built (python -m fused3s_amd.build); there is no fallback")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        L.f3s_abi_version.restype = ci
+        L.f3s_last_error.restype = ctypes.c_char_p
+        L.f3s_preprocess_workspace_bytes.restype = cs
+        L.f3s_preprocess_workspace_bytes.argtypes = [ci, ci]
+        L.f3s_preprocess_count.restype = ci
+        L.f3s_preprocess_count.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, cs,
+                                           ctypes.POINTER(ctypes.c_int64), vp]
+        L.f3s_preprocess_fill.restype = ci
+        L.f3s_preprocess_fill.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, ctypes.c_int64, vp, vp,
+                                          vp, vp, vp, vp]
+        L.f3s_attention_fwd.restype = ci
+        L.f3s_attention_fwd.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, vp, ctypes.c_float,
+                                        ci, vp, vp, vp]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError("libf3s_amd: %s (status %d)" % (lib().f3s_last_error().decode(), rc))
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, dtype, name):
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a device tensor" % name)
+    if t.dtype != dtype:
+        raise RuntimeError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+
+
+def preprocess(rowPtr, colIdx, N, H=16, W=16):
+    """Both preprocessing phases through the C ABI. Returns a dict of device tensors."""
+    L = lib()
+    _dev(rowPtr, torch.int32, "rowPtr")
+    _dev(colIdx, torch.int32, "colIdx")
+    dev = rowPtr.device
+    E = int(colIdx.numel())
+    nRW = (N + H - 1) // H
+    i32 = dict(dtype=torch.int32, device=dev)
+    blockPartition = torch.empty(nRW, **i32)
+    edgeToColumn = torch.empty(E, **i32)
+    edgeToRow = torch.empty(E, **i32)
+    rwo = torch.empty(nRW + 1, **i32)
+    order = torch.empty(nRW, **i32)
+    wsBytes = L.f3s_preprocess_workspace_bytes(N, E)
+    ws = torch.empty(wsBytes, dtype=torch.uint8, device=dev)
+    nTcb = ctypes.c_int64(-1)
+    with torch.cuda.device(dev):
+        _check(L.f3s_preprocess_count(_ptr(rowPtr), _ptr(colIdx), N, E, H, W,
+                                      _ptr(blockPartition), _ptr(edgeToColumn), _ptr(edgeToRow),
+                                      _ptr(rwo), _ptr(order), _ptr(ws), wsBytes,
+                                      ctypes.byref(nTcb), _stream()))
+        nT = int(nTcb.value)
+        rowid = torch.empty(nT, **i32)
+        tile = torch.empty(E, dtype=torch.uint8, device=dev)
+        toff = torch.empty(nT + 1, **i32)
+        atox = torch.empty(nT * W, **i32)
+        bm = torch.empty(nT * H * W // 64, dtype=torch.uint64, device=dev)
+        _check(L.f3s_preprocess_fill(_ptr(rowPtr), _ptr(colIdx), N, E, H, W, _ptr(edgeToColumn),
+                                     _ptr(rwo), nT, _ptr(rowid), _ptr(tile), _ptr(toff),
+                                     _ptr(atox), _ptr(bm), _stream()))
+    return dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
+                tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox, tcbBitMap=bm,
+                blockCount=nT, blockPartition=blockPartition, edgeToColumn=edgeToColumn,
+                edgeToRow=edgeToRow)
+
+
+def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoftmax=True,
+              out=None):
+    """f3s_attention_fwd on the current stream; returns out fp32[N, d]."""
+    L = lib()
+    _dev(rwo, torch.int32, "rowWindowOffset")
+    _dev(atox, torch.int32, "sparseAToXidx")
+    _dev(bitmap, torch.uint64, "tcbBitMap")
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        _dev(t, Q.dtype, name)
+    if order is not None:
+        _dev(order, torch.int32, "windowOrder")
+    if Q.dtype == torch.float16:
+        dtype = 0
+    elif Q.dtype == torch.bfloat16:
+        dtype = 1
+    else:
+        raise RuntimeError("Q/K/V must be float16 or bfloat16")
+    d = Q.shape[1]
+    if Q.shape[0] < N or K.shape != Q.shape or V.shape != Q.shape:
+        raise RuntimeError("Q/K/V must be [N, d] with identical shapes")
+    if rwo.numel() != (N + 15) // 16 + 1:
+        raise RuntimeError("rowWindowOffset has %d entries, expected %d"
+                           % (rwo.numel(), (N + 15) // 16 + 1))
+    if order is not None and order.numel() != rwo.numel() - 1:
+        raise RuntimeError("windowOrder must have one entry per row window")
+    if out is None:
+        out = torch.empty((N, d), dtype=torch.float32, device=Q.device)
+    with torch.cuda.device(Q.device):
+        _check(L.f3s_attention_fwd(_ptr(rwo), _ptr(order), _ptr(atox), _ptr(bitmap), N, d, dtype,
+                                   _ptr(Q), _ptr(K), _ptr(V), float(scalingFactor),
+                                   int(bool(applySoftmax)), _ptr(out), None, _stream()))
+    return out

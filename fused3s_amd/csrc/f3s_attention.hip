@@ -1,0 +1,283 @@
+// Fused SDDMM -> online softmax -> SpMM over 16x16 TC blocks for gfx950 (MI355X), wave64.
+//
+// Replaces the reference kernels f3sKernel1tb1rw / ...Scheduled / ...ScheduledPermutedQKV
+// [ScaleQK] and f2sKernel1tb1rw (src/F3S_kernel.cu:997-1175, 1371-1800, 1999-2182, 2186-2327)
+// and their launchers (src/F3S_kernel.cu:393-458, 581-671).
+//
+// One workgroup owns one 16-row window; its waves take the window's TC blocks two at a time
+// (pair p -> wave p % NWAVES) and keep private running (m, l, O) in registers. One LDS merge
+// per window combines the waves (log-sum-exp), instead of the reference's three block barriers
+// per iteration.
+//
+// Register dataflow of one TC-block pair (lane = 16*g + c, g in 0..3, c in 0..15):
+//   S^T = K_t Q^T   v_mfma_f32_16x16x32_f16, A = gathered K rows (lane: row slot c, features
+//                   32i+8g..+7, one 16-byte load), B = Q (lane: query row c, same features).
+//                   The accumulator leaves S[q=c][slot 4g+i], i<4, in this lane.
+//   mask            one byte of the block's bitmap holds this lane's 4 bits.
+//   softmax         row q=c lives in lanes c, c+16, c+32, c+48: 8 in-register values and two
+//                   cross-lane steps.
+//   O^T += V^T P^T  v_mfma_f32_16x16x32_f16 over the 32 keys of the pair, contraction index
+//                   8g+k <-> (block A, slot 4g+k) for k<4, (block B, slot 4g+k-4) for k>=4, so
+//                   the B operand is exactly the 8 probabilities this lane already holds.
+//                   A = V^T: the lane reads D/16 contiguous halfs of each of its 8 key rows
+//                   (16 lanes cover one whole V row: coalesced), element j feeds output tile j.
+//                   Tile j therefore owns output columns {c*(D/16)+j}; after the MFMA lane
+//                   (g,c) holds O[q=c][g*D/4 .. (g+1)*D/4), a contiguous run.
+// Neither Q, K, V nor P touches LDS.
+//
+// Numerics follow the reference kernel (src/F3S_kernel.cu:1402-1406,1447-1451,1487-1499,
+// 938-945,1560-1561): running max starts at 0 and masked zeros take part in it, an unmasked
+// score that is exactly 0 is dropped like a masked one, the row sum uses un-rounded fp32
+// exponentials while P is rounded to fp16 for the second MFMA, empty rows give 0.
+#include "f3s_common.h"
+
+namespace f3s {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <int T>
+struct HalfVec {
+  typedef _Float16 type __attribute__((ext_vector_type(T)));
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max / sum over the four lanes {c, c+16, c+32, c+48} that share a query row
+__device__ __forceinline__ float row_max4(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16));
+  v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+__device__ __forceinline__ float row_sum4(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+template <int D, int NWAVES, bool SOFTMAX>
+__global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
+    const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
+    const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
+    const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+    const _Float16* __restrict__ V, float scaleLog2, float* __restrict__ out) {
+  constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
+  constexpr int KS = D / 32;  // MFMA k-steps of the score product
+  constexpr int OSTRIDE = D + 4;
+  typedef typename HalfVec<T>::type vrow_t;
+
+  __shared__ float sM[NWAVES][16];
+  __shared__ float sL[NWAVES][16];
+  __shared__ float sO[NWAVES][16][OSTRIDE];
+
+  const int w = windowOrder ? windowOrder[blockIdx.x] : (int)blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const int t0 = rowWindowOffset[w];
+  const int t1 = rowWindowOffset[w + 1];
+  const int nPairs = (t1 - t0 + 1) >> 1;
+
+  // B operand of the score product: this lane's query row, features 32i + 8g .. +7
+  half8 qf[KS];
+  {
+    const int64_t qrow = (int64_t)w * 16 + c;
+    if (qrow < N) {
+      const half8* qp = reinterpret_cast<const half8*>(Q + qrow * D) + g;
+#pragma unroll
+      for (int i = 0; i < KS; i++) qf[i] = qp[4 * i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < KS; i++) qf[i] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+
+  float m = 0.0f;  // running row max (log2 domain when SOFTMAX), starts at 0 like the reference
+  float l = 0.0f;  // this lane's share of the row sum
+  float4v o[T];
+#pragma unroll
+  for (int j = 0; j < T; j++) o[j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  const int maskByte = ((g >> 1) * 2 + (c >> 3)) * 8 + 7 - (c & 7);
+  const int maskShift = 4 * (1 - (g & 1));
+
+  for (int p = wave; p < nPairs; p += NWAVES) {
+    const int tA = t0 + 2 * p;
+    const bool hasB = (tA + 1) < t1;
+    const int tB = hasB ? tA + 1 : tA;
+
+    // gathered K rows -> A operand
+    const int kRowA = sparseAToXidx[tA * 16 + c];
+    const int kRowB = sparseAToXidx[tB * 16 + c];
+    const half8* kpA = reinterpret_cast<const half8*>(K + (int64_t)kRowA * D) + g;
+    const half8* kpB = reinterpret_cast<const half8*>(K + (int64_t)kRowB * D) + g;
+    half8 kA[KS], kB[KS];
+#pragma unroll
+    for (int i = 0; i < KS; i++) {
+      kA[i] = kpA[4 * i];
+      kB[i] = kpB[4 * i];
+    }
+    // V rows of this lane's 8 contraction slots
+    const int4 vIdxA = reinterpret_cast<const int4*>(sparseAToXidx + tA * 16)[g];
+    const int4 vIdxB = reinterpret_cast<const int4*>(sparseAToXidx + tB * 16)[g];
+    const int vr[8] = {vIdxA.x, vIdxA.y, vIdxA.z, vIdxA.w, vIdxB.x, vIdxB.y, vIdxB.z, vIdxB.w};
+    vrow_t vv[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++)
+      vv[k] = reinterpret_cast<const vrow_t*>(V + (int64_t)vr[k] * D)[c];
+
+    unsigned bitsA = (bitmapBytes[(int64_t)tA * 32 + maskByte] >> maskShift) & 0xFu;
+    unsigned bitsB = (bitmapBytes[(int64_t)tB * 32 + maskByte] >> maskShift) & 0xFu;
+    if (!hasB) bitsB = 0;
+
+    float4v sA = {0.f, 0.f, 0.f, 0.f}, sB = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KS; i++) {
+      sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kA[i], qf[i], sA, 0, 0, 0);
+      sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kB[i], qf[i], sB, 0, 0, 0);
+    }
+    float s[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      s[i] = ((bitsA >> (3 - i)) & 1u) ? sA[i] : 0.0f;
+      s[4 + i] = ((bitsB >> (3 - i)) & 1u) ? sB[i] : 0.0f;
+    }
+
+    half8 pf;
+    if constexpr (SOFTMAX) {
+      float mx = m;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        s[i] *= scaleLog2;
+        mx = fmaxf(mx, s[i]);
+      }
+      mx = row_max4(mx);
+      const float alpha = fast_exp2(m - mx);
+      m = mx;
+      float sum = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const float e = (s[i] == 0.0f) ? 0.0f : fast_exp2(s[i] - mx);
+        sum += e;
+        pf[i] = (_Float16)e;
+      }
+      l = fmaf(alpha, l, sum);
+#pragma unroll
+      for (int j = 0; j < T; j++) o[j] *= alpha;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) pf[i] = (_Float16)s[i];
+    }
+
+#pragma unroll
+    for (int j = 0; j < T; j++) {
+      half8 va;
+#pragma unroll
+      for (int k = 0; k < 8; k++) va[k] = vv[k][j];
+      o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pf, o[j], 0, 0, 0);
+    }
+  }
+
+  // ---- merge the waves' partial (m, l, O) and write the window's rows
+  if constexpr (SOFTMAX) l = row_sum4(l);
+  if (g == 0) {
+    sM[wave][c] = m;
+    sL[wave][c] = l;
+  }
+#pragma unroll
+  for (int j = 0; j < T; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) sO[wave][c][g * (D / 4) + i * T + j] = o[j][i];
+  __syncthreads();
+
+  constexpr int VEC_PER_ROW = D / 4;
+  for (int idx = threadIdx.x; idx < 16 * VEC_PER_ROW; idx += NWAVES * 64) {
+    const int q = idx / VEC_PER_ROW;
+    const int cv = idx % VEC_PER_ROW;
+    const int64_t row = (int64_t)w * 16 + q;
+    if (row >= N) continue;
+    float4 acc = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (SOFTMAX) {
+      float mAll = sM[0][q];
+#pragma unroll
+      for (int v = 1; v < NWAVES; v++) mAll = fmaxf(mAll, sM[v][q]);
+      float lAll = 0.0f;
+#pragma unroll
+      for (int v = 0; v < NWAVES; v++) {
+        const float f = fast_exp2(sM[v][q] - mAll);
+        lAll = fmaf(f, sL[v][q], lAll);
+        const float4 ov = *reinterpret_cast<const float4*>(&sO[v][q][cv * 4]);
+        acc.x = fmaf(f, ov.x, acc.x);
+        acc.y = fmaf(f, ov.y, acc.y);
+        acc.z = fmaf(f, ov.z, acc.z);
+        acc.w = fmaf(f, ov.w, acc.w);
+      }
+      const float inv = (lAll == 0.0f) ? 0.0f : 1.0f / lAll;
+      acc.x *= inv;
+      acc.y *= inv;
+      acc.z *= inv;
+      acc.w *= inv;
+    } else {
+#pragma unroll
+      for (int v = 0; v < NWAVES; v++) {
+        const float4 ov = *reinterpret_cast<const float4*>(&sO[v][q][cv * 4]);
+        acc.x += ov.x;
+        acc.y += ov.y;
+        acc.z += ov.z;
+        acc.w += ov.w;
+      }
+    }
+    *reinterpret_cast<float4*>(out + row * D + cv * 4) = acc;
+  }
+}
+
+template <int D, bool SOFTMAX>
+int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, const uint64_t* bitmap,
+             int N, const void* Q, const void* K, const void* V, float scaleLog2, float* out,
+             hipStream_t stream) {
+  constexpr int NWAVES = 4;
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  if (nRW == 0) return 0;
+  hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX>), dim3(nRW), dim3(NWAVES * 64), 0, stream,
+                     rwo, order, atox, reinterpret_cast<const uint8_t*>(bitmap), N,
+                     static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
+                     static_cast<const _Float16*>(V), scaleLog2, out);
+  F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+
+int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                     int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
+                     int applySoftmax, float* out, unsigned long long* cuTimer,
+                     hipStream_t stream) {
+  if (dtype != 0) return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16)", dtype);
+  if (cuTimer) return fail(-3, "f3s_attention_fwd: per-CU timing not supported yet");
+  if (scalingFactor == 0.0f) return fail(-2, "f3s_attention_fwd: scalingFactor must be non-zero");
+  // the reference divides unmasked scores by scalingFactor (src/F3S_kernel.cu:1666-1667);
+  // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
+  const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
+#define F3S_DISPATCH(DD)                                                                       \
+  case DD:                                                                                     \
+    return applySoftmax ? launch_d<DD, true>(rowWindowOffset, windowOrder, sparseAToXidx,      \
+                                             bitmap, N, Q, K, V, scaleLog2, out, stream)       \
+                        : launch_d<DD, false>(rowWindowOffset, windowOrder, sparseAToXidx,     \
+                                              bitmap, N, Q, K, V, scaleLog2, out, stream);
+  switch (d) {
+    F3S_DISPATCH(32)
+    F3S_DISPATCH(64)
+    F3S_DISPATCH(128)
+    default:
+      return fail(-2, "f3s_attention_fwd: head dim %d unsupported (32, 64, 128)", d);
+  }
+#undef F3S_DISPATCH
+}
+
+}  // namespace f3s

@@ -1,0 +1,89 @@
+// C ABI of libf3s_amd.so (declared in include/f3s_amd.h): argument checks, error text,
+// dispatch into the HIP launchers.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/f3s_amd.h"
+#include "f3s_common.h"
+
+namespace f3s {
+namespace {
+thread_local char g_error[512] = "";
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+namespace {
+bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+}  // namespace
+}  // namespace f3s
+
+extern "C" {
+
+int f3s_abi_version(void) { return 1; }
+
+const char* f3s_last_error(void) { return f3s::g_error; }
+
+size_t f3s_preprocess_workspace_bytes(int N, int E) {
+  if (N < 0) N = 0;
+  return f3s::preprocess_workspace_bytes(N, E);
+}
+
+int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                         int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                         int32_t* rowWindowOffset, int32_t* sortedRowWindows, void* workspace,
+                         size_t ws_bytes, int64_t* nTCB_host, void* stream) {
+  if (!rowPtr || !rowWindowOffset || !workspace || !nTCB_host)
+    return f3s::fail(-1, "f3s_preprocess_count: null pointer");
+  if (N > 0 && (!blockPartition || !sortedRowWindows))
+    return f3s::fail(-1, "f3s_preprocess_count: null window output");
+  if (E > 0 && (!colIdx || !edgeToColumn || !edgeToRow))
+    return f3s::fail(-1, "f3s_preprocess_count: null edge array");
+  if (f3s::misaligned(workspace, 256))
+    return f3s::fail(-1, "f3s_preprocess_count: workspace must be 256-byte aligned");
+  return f3s::launch_preprocess_count(rowPtr, colIdx, N, E, H, W, blockPartition, edgeToColumn,
+                                      edgeToRow, rowWindowOffset, sortedRowWindows, workspace,
+                                      ws_bytes, nTCB_host, static_cast<hipStream_t>(stream));
+}
+
+int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                        const int32_t* edgeToColumn, const int32_t* rowWindowOffset, int64_t nTCB,
+                        int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                        int32_t* sparseAToXidx, uint64_t* tcbBitMap, void* stream) {
+  if (!rowPtr || !rowWindowOffset || !tcblockOffset)
+    return f3s::fail(-1, "f3s_preprocess_fill: null pointer");
+  if (nTCB < 0 || N < 0 || E < 0) return f3s::fail(-2, "f3s_preprocess_fill: negative size");
+  if (nTCB > 0 && (!tcblockRowid || !sparseAToXidx || !tcbBitMap || !colIdx || !edgeToColumn ||
+                   !tcblocktileId))
+    return f3s::fail(-1, "f3s_preprocess_fill: null output");
+  if (f3s::misaligned(tcbBitMap, 8))
+    return f3s::fail(-1, "f3s_preprocess_fill: tcbBitMap must be 8-byte aligned");
+  return f3s::launch_preprocess_fill(rowPtr, colIdx, N, E, H, W, edgeToColumn, rowWindowOffset,
+                                     nTCB, tcblockRowid, tcblocktileId, tcblockOffset,
+                                     sparseAToXidx, tcbBitMap, static_cast<hipStream_t>(stream));
+}
+
+int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int d,
+                      int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
+                      int applySoftmax, float* out, unsigned long long* cuTimer, void* stream) {
+  if (N < 0) return f3s::fail(-2, "f3s_attention_fwd: negative N");
+  if (N == 0) return 0;
+  if (!rowWindowOffset || !Q || !K || !V || !out)
+    return f3s::fail(-1, "f3s_attention_fwd: null pointer");
+  if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
+      f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
+      f3s::misaligned(tcbBitMap, 8))
+    return f3s::fail(-1, "f3s_attention_fwd: Q/K/V/out/sparseAToXidx need 16-byte alignment");
+  return f3s::launch_attention(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, d,
+                               dtype, Q, K, V, scalingFactor, applySoftmax, out, cuTimer,
+                               static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+// Shared declarations of the MI355X Fused3S library (internal; the public C ABI is
+// include/f3s_amd.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace f3s {
+
+constexpr int kWave = 64;       // CDNA4 wavefront width
+constexpr int kWinRows = 16;    // rows per row window (reference BLK_H / BLK_M)
+
+// Records a message retrievable through f3s_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+#define F3S_HIP_CHECK(expr)                                                          \
+  do {                                                                               \
+    hipError_t e__ = (expr);                                                         \
+    if (e__ != hipSuccess)                                                           \
+      return ::f3s::fail(-100, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__), \
+                         __FILE__, __LINE__);                                        \
+  } while (0)
+
+// attention (f3s_attention.hip)
+int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                     int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
+                     int applySoftmax, float* out, unsigned long long* cuTimer,
+                     hipStream_t stream);
+
+// preprocessing (f3s_preprocess.hip)
+size_t preprocess_workspace_bytes(int N, int E);
+int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                            int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                            int32_t* edgeToRow, int32_t* rowWindowOffset,
+                            int32_t* sortedRowWindows, void* workspace, size_t wsBytes,
+                            int64_t* nTcbHost, hipStream_t stream);
+int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                           int W, const int32_t* edgeToColumn, const int32_t* rowWindowOffset,
+                           int64_t nTcb, int32_t* tcblockRowid, uint8_t* tcblocktileId,
+                           int32_t* tcblockOffset, int32_t* sparseAToXidx, uint64_t* bitmap,
+                           hipStream_t stream);
+
+}  // namespace f3s

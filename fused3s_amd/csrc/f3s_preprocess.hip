@@ -1,0 +1,477 @@
+// CSR -> 16-row windows of column-compacted TC blocks with per-block bitmaps, on gfx950.
+//
+// Replaces the reference's preprocessing pipeline (src/F3S.cpp:40-87, src/utils.cu:23-436):
+// a global thrust::sort of (window, column) pairs followed by two kernels that walk each
+// window with a single thread. Here a window never leaves its workgroup:
+//
+//   window_rank_kernel   one workgroup per window. Column ids are OR-ed into an LDS bitset
+//                        (a column range per pass when N exceeds the LDS range), a wave64
+//                        popcount prefix scan turns the bitset into ranks, and every edge
+//                        reads its compacted column index back: the sorted unique column list
+//                        (reference: sort + inplace_deduplication + binarysearch,
+//                        src/utils.cu:102-153,281-289) is never materialised.
+//   finalize_count_kernel one workgroup: inclusive scan of the per-window block counts
+//                        (src/utils.cu:293-300) and a stable LSD radix sort of the windows by
+//                        descending block count (src/utils.cu:400-436), ranks from wave ballots.
+//   window_fill_kernel   one workgroup per window: bitmaps and per-(row, block) edge counts are
+//                        accumulated in LDS, a block-wide scan yields the per-block offsets, and
+//                        each wave replays its rows in CSR order to place the tile ids
+//                        (src/utils.cu:173-224, 23-36, 53-65).
+//
+// All results are bit-identical to the reference's algorithm with edgeToRow[e] = row(e).
+#include "f3s_common.h"
+
+namespace f3s {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kRangeMax = 393216;  // columns per bitset pass: 48 KiB of bits + 12 KiB of prefixes
+constexpr int kFillChunk = 512;    // TC blocks held in LDS at once by window_fill_kernel
+
+// workspace header (bytes 0..255): int64 nTCB, int32 error flag
+struct WsHeader {
+  long long nTcb;
+  int error;
+};
+constexpr size_t kWsHeaderBytes = 256;
+
+__device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    unsigned n = __shfl_up(v, off);
+    if (lane >= off) v += n;
+  }
+  return v;
+}
+
+// largest r in [0,15] with sRow[r] <= e (sRow[0] <= e < sRow[16])
+__device__ __forceinline__ int row_of_edge(const int* sRow, int e) {
+  int r = 0;
+  if (sRow[r + 8] <= e) r += 8;
+  if (sRow[r + 4] <= e) r += 4;
+  if (sRow[r + 2] <= e) r += 2;
+  if (sRow[r + 1] <= e) r += 1;
+  return r;
+}
+
+// ------------------------------------------------------------------ phase 1
+template <int W>
+__global__ __launch_bounds__(kBlock) void window_rank_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
+    int nPasses, int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr) {
+  extern __shared__ __align__(16) uint32_t smem[];
+  uint32_t* bits = smem;                 // range/32 words
+  uint32_t* pref = smem + (range >> 5);  // range/128 group prefixes
+  __shared__ int sRow[17];
+  __shared__ unsigned sWaveTot[kBlock / 64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int w = blockIdx.x;
+  const int r0 = w * 16;
+  if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
+  __syncthreads();
+  const int eS = sRow[0], eE = sRow[16];
+  if (eS == eE) {
+    if (tid == 0) blockPartition[w] = 0;
+    return;
+  }
+  const int nGroups = range >> 7;
+  unsigned uniqueBefore = 0;
+  for (int pass = 0; pass < nPasses; pass++) {
+    const int lo = pass * range;
+    for (int i = tid; i < nGroups; i += kBlock)
+      reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+    for (int e = eS + tid; e < eE; e += kBlock) {
+      const int col = colIdx[e];
+      if ((unsigned)col >= (unsigned)N) {
+        atomicOr(&hdr->error, 1);
+        continue;
+      }
+      const unsigned rel = (unsigned)(col - lo);
+      if (rel < (unsigned)range) atomicOr(&bits[rel >> 5], 1u << (rel & 31));
+    }
+    __syncthreads();
+    unsigned carry = uniqueBefore;
+    for (int gb = 0; gb < nGroups; gb += kBlock) {
+      const int gi = gb + tid;
+      unsigned cnt = 0;
+      if (gi < nGroups) {
+        const uint4 v = reinterpret_cast<const uint4*>(bits)[gi];
+        cnt = __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+      }
+      const unsigned incl = wave_inclusive_scan(cnt, lane);
+      if (lane == 63) sWaveTot[wave] = incl;
+      __syncthreads();
+      unsigned waveOff = 0, tileTot = 0;
+#pragma unroll
+      for (int v = 0; v < kBlock / 64; v++) {
+        const unsigned t = sWaveTot[v];
+        if (v < wave) waveOff += t;
+        tileTot += t;
+      }
+      if (gi < nGroups) pref[gi] = carry + waveOff + incl - cnt;
+      carry += tileTot;
+      __syncthreads();
+    }
+    for (int e = eS + tid; e < eE; e += kBlock) {
+      const int col = colIdx[e];
+      const unsigned rel = (unsigned)(col - lo);
+      if ((unsigned)col < (unsigned)N && rel < (unsigned)range) {
+        const unsigned wd = rel >> 5;
+        unsigned rank = pref[wd >> 2];
+        for (unsigned k = wd & ~3u; k < wd; k++) rank += __popc(bits[k]);
+        rank += __popc(bits[wd] & ((1u << (rel & 31)) - 1u));
+        edgeToColumn[e] = (int)rank;
+      }
+    }
+    uniqueBefore = carry;
+    __syncthreads();
+  }
+  for (int e = eS + tid; e < eE; e += kBlock) edgeToRow[e] = r0 + row_of_edge(sRow, e);
+  if (tid == 0) blockPartition[w] = (int)((uniqueBefore + W - 1) / W);
+}
+
+// ------------------------------------------------- scan + window ordering
+constexpr int kFinBlock = 1024;
+
+__global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
+    const int32_t* __restrict__ blockPartition, int nRW, int32_t* __restrict__ rowWindowOffset,
+    int32_t* __restrict__ sortedRowWindows, int32_t* __restrict__ keysA,
+    int32_t* __restrict__ keysB, int32_t* __restrict__ valsTmp, WsHeader* __restrict__ hdr) {
+  constexpr int NW = kFinBlock / 64;
+  __shared__ unsigned sWave[NW];
+  __shared__ int sMax;
+  __shared__ unsigned sBinBase[16];
+  __shared__ unsigned sCnt[NW][16];
+  __shared__ unsigned sOff[NW][16];
+  __shared__ unsigned sTileTot[16];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+
+  // inclusive scan of the block counts into rowWindowOffset[1..], and their maximum
+  if (tid == 0) sMax = 0;
+  __syncthreads();
+  unsigned carry = 0;
+  int localMax = 0;
+  for (int base = 0; base < nRW; base += kFinBlock) {
+    const int i = base + tid;
+    const unsigned v = (i < nRW) ? (unsigned)blockPartition[i] : 0u;
+    localMax = max(localMax, (int)v);
+    const unsigned incl = wave_inclusive_scan(v, lane);
+    if (lane == 63) sWave[wave] = incl;
+    __syncthreads();
+    unsigned waveOff = 0, tot = 0;
+#pragma unroll
+    for (int k = 0; k < NW; k++) {
+      const unsigned t = sWave[k];
+      if (k < wave) waveOff += t;
+      tot += t;
+    }
+    if (i < nRW) rowWindowOffset[i + 1] = (int)(carry + waveOff + incl);
+    carry += tot;
+    __syncthreads();
+  }
+  atomicMax(&sMax, localMax);
+  if (tid == 0) {
+    rowWindowOffset[0] = 0;
+    hdr->nTcb = (long long)carry;
+  }
+  __syncthreads();
+  const int maxC = sMax;
+
+  // stable sort by descending count == stable ascending LSD radix sort of (maxC - count)
+  int nBits = 0;
+  while ((maxC >> nBits) != 0) nBits++;
+  const int nPass = (nBits + 3) / 4;
+  if (nPass == 0) {
+    for (int i = tid; i < nRW; i += kFinBlock) sortedRowWindows[i] = i;
+    return;
+  }
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  for (int pass = 0; pass < nPass; pass++) {
+    const int shift = pass * 4;
+    const bool toOut = ((nPass - 1 - pass) & 1) == 0;
+    int32_t* kDst = toOut ? keysA : keysB;
+    int32_t* vDst = toOut ? sortedRowWindows : valsTmp;
+    const int32_t* kSrc = toOut ? keysB : keysA;
+    const int32_t* vSrc = toOut ? valsTmp : sortedRowWindows;
+    if (tid < 16) sBinBase[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < nRW; i += kFinBlock) {
+      const int key = (pass == 0) ? (maxC - blockPartition[i]) : kSrc[i];
+      atomicAdd(&sBinBase[(key >> shift) & 15], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      unsigned run = 0;
+      for (int dgt = 0; dgt < 16; dgt++) {
+        const unsigned c = sBinBase[dgt];
+        sBinBase[dgt] = run;
+        run += c;
+      }
+    }
+    __syncthreads();
+    for (int base = 0; base < nRW; base += kFinBlock) {
+      const int i = base + tid;
+      const bool valid = i < nRW;
+      int key = 0, val = 0;
+      if (valid) {
+        key = (pass == 0) ? (maxC - blockPartition[i]) : kSrc[i];
+        val = (pass == 0) ? i : vSrc[i];
+      }
+      const int dgt = (key >> shift) & 15;
+      if (tid < NW * 16) (&sCnt[0][0])[tid] = 0;
+      __syncthreads();
+      unsigned long long peers = __ballot(valid);
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const unsigned long long bal = __ballot((dgt >> b) & 1);
+        peers &= ((dgt >> b) & 1) ? bal : ~bal;
+      }
+      const unsigned rank = __popcll(peers & ltMask);
+      if (valid && rank == 0) sCnt[wave][dgt] = __popcll(peers);
+      __syncthreads();
+      if (tid < NW * 16) {
+        const int d2 = tid & 15, v2 = tid >> 4;
+        unsigned off = 0;
+        for (int k = 0; k < v2; k++) off += sCnt[k][d2];
+        sOff[v2][d2] = off;
+        if (v2 == NW - 1) sTileTot[d2] = off + sCnt[v2][d2];
+      }
+      __syncthreads();
+      if (valid) {
+        const unsigned pos = sBinBase[dgt] + sOff[wave][dgt] + rank;
+        kDst[pos] = key;
+        vDst[pos] = val;
+      }
+      __syncthreads();
+      if (tid < 16) sBinBase[tid] += sTileTot[tid];
+      __syncthreads();
+    }
+  }
+}
+
+// ------------------------------------------------------------------ phase 2
+template <int W>
+__global__ __launch_bounds__(kBlock) void window_fill_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
+    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
+    long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
+    int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
+    unsigned long long* __restrict__ bitmap) {
+  constexpr int TC = kFillChunk;
+  constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
+  constexpr int LOGW = (W == 16) ? 4 : 3;
+  __shared__ unsigned sCnt[TC * 16];            // [block][row] counts, then running positions
+  __shared__ unsigned long long sBm[TC * WPT];  // bitmaps of the chunk
+  __shared__ int sRow[17];
+  __shared__ unsigned sWaveTot[kBlock / 64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int w = blockIdx.x;
+  if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
+  const int base = rowWindowOffset[w];
+  const int nb = rowWindowOffset[w + 1] - base;
+  if (nb == 0) return;
+  const int r0 = w * 16;
+  if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
+  __syncthreads();
+  const int eS = sRow[0], eE = sRow[16];
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  unsigned carry = (unsigned)eS;  // absolute edge position where the next TC block starts
+
+  for (int tc0 = 0; tc0 < nb; tc0 += TC) {
+    const int nt = min(TC, nb - tc0);
+    for (int i = tid; i < nt * 16; i += kBlock) sCnt[i] = 0;
+    for (int i = tid; i < nt * WPT; i += kBlock) sBm[i] = 0ull;
+    __syncthreads();
+    for (int e = eS + tid; e < eE; e += kBlock) {
+      const int ec = edgeToColumn[e];
+      const int t = (ec >> LOGW) - tc0;
+      if ((unsigned)t < (unsigned)nt) {
+        const int r = row_of_edge(sRow, e);
+        const int cl = ec & (W - 1);
+        atomicAdd(&sCnt[t * 16 + r], 1u);
+        // 8x8 sub-blocks in column-major order, row-major and MSB-first inside
+        const int sub = (cl >> 3) * (W / 8) + (r >> 3);
+        atomicOr(&sBm[t * WPT + sub], 1ull << (63 - ((r & 7) * 8 + (cl & 7))));
+        sparseAToXidx[(int64_t)(base + tc0 + t) * W + cl] = colIdx[e];
+      }
+    }
+    __syncthreads();
+    for (int tb = 0; tb < nt; tb += kBlock) {
+      const int t = tb + tid;
+      unsigned nnz = 0;
+      if (t < nt) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) nnz += sCnt[t * 16 + r];
+      }
+      const unsigned incl = wave_inclusive_scan(nnz, lane);
+      if (lane == 63) sWaveTot[wave] = incl;
+      __syncthreads();
+      unsigned waveOff = 0, tileTot = 0;
+#pragma unroll
+      for (int v = 0; v < kBlock / 64; v++) {
+        const unsigned x = sWaveTot[v];
+        if (v < wave) waveOff += x;
+        tileTot += x;
+      }
+      if (t < nt) {
+        const int64_t gt = (int64_t)base + tc0 + t;
+        unsigned run = carry + waveOff + incl - nnz;
+        tcblockOffset[gt] = (int)run;
+        tcblockRowid[gt] = w;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const unsigned c = sCnt[t * 16 + r];
+          sCnt[t * 16 + r] = run;
+          run += c;
+        }
+        // bitmap words out; a compacted slot that no edge named keeps column id 0
+        unsigned colMask = 0;  // bit cl set <=> slot cl holds a column
+#pragma unroll
+        for (int k = 0; k < WPT; k++) {
+          const unsigned long long word = sBm[t * WPT + k];
+          bitmap[gt * WPT + k] = word;
+          unsigned long long x = word;
+          x |= x >> 32;
+          x |= x >> 16;
+          x |= x >> 8;
+          const unsigned rowOr = (unsigned)(x & 0xFFull);  // bit (7 - cl%8)
+          const int colHalf = (W == 16) ? (k >> 1) : 0;
+#pragma unroll
+          for (int b = 0; b < 8; b++)
+            if (rowOr & (0x80u >> b)) colMask |= 1u << (colHalf * 8 + b);
+        }
+#pragma unroll
+        for (int cl = 0; cl < W; cl++)
+          if (!((colMask >> cl) & 1u)) sparseAToXidx[gt * W + cl] = 0;
+      }
+      carry += tileTot;
+      __syncthreads();
+    }
+    // tile ids: each wave replays whole rows in CSR order, so positions inside a TC block
+    // follow the edge order (src/utils.cu:213-223)
+    for (int r = wave; r < 16; r += kBlock / 64) {
+      const int rs = sRow[r], re = sRow[r + 1];
+      for (int eb = rs; eb < re; eb += 64) {
+        const int e = eb + lane;
+        const bool valid = e < re;
+        const int ec = valid ? edgeToColumn[e] : 0;
+        const int t = (ec >> LOGW) - tc0;
+        const bool inr = valid && (unsigned)t < (unsigned)nt;
+        unsigned long long peers = __ballot(inr);
+        if (peers == 0ull) continue;
+#pragma unroll
+        for (int b = 0; b < 9; b++) {
+          const unsigned long long bal = __ballot((t >> b) & 1);
+          peers &= ((t >> b) & 1) ? bal : ~bal;
+        }
+        unsigned pos = 0;
+        if (inr) pos = sCnt[t * 16 + r] + __popcll(peers & ltMask);
+        if (inr) tcblocktileId[pos] = (uint8_t)(r * W + (ec & (W - 1)));
+        // the highest peer lane advances the running position of (block, row)
+        if (inr && (peers >> lane) == 1ull) sCnt[t * 16 + r] += __popcll(peers);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+__global__ void set_tail_kernel(int32_t* tcblockOffset, long long nTcb, int E) {
+  tcblockOffset[nTcb] = E;
+}
+
+__global__ void clear_header_kernel(WsHeader* hdr) {
+  hdr->nTcb = 0;
+  hdr->error = 0;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace
+
+size_t preprocess_workspace_bytes(int N, int /*E*/) {
+  const size_t nRW = (size_t)(N + kWinRows - 1) / kWinRows;
+  return kWsHeaderBytes + 3 * align256(nRW * sizeof(int32_t));
+}
+
+int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                            int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                            int32_t* edgeToRow, int32_t* rowWindowOffset,
+                            int32_t* sortedRowWindows, void* workspace, size_t wsBytes,
+                            int64_t* nTcbHost, hipStream_t stream) {
+  if (H != 16 || (W != 16 && W != 8))
+    return fail(-2, "f3s_preprocess_count: block %dx%d unsupported (16x16 or 16x8)", H, W);
+  if (N < 0 || E < 0) return fail(-2, "f3s_preprocess_count: negative size");
+  if (wsBytes < preprocess_workspace_bytes(N, E))
+    return fail(-2, "f3s_preprocess_count: workspace %zu B < required %zu B", wsBytes,
+                preprocess_workspace_bytes(N, E));
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  char* ws = static_cast<char*>(workspace);
+  WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
+  const size_t seg = align256((size_t)nRW * sizeof(int32_t));
+  int32_t* keysA = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes);
+  int32_t* keysB = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + seg);
+  int32_t* valsTmp = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + 2 * seg);
+
+  hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(1), 0, stream, hdr);
+  if (nRW > 0) {
+    int range = ((N + 127) / 128) * 128;
+    if (range > kRangeMax) range = kRangeMax;
+    const int nPasses = (N + range - 1) / range;
+    const size_t lds = (size_t)(range / 32 + range / 128) * sizeof(uint32_t);
+    if (W == 16)
+      hipLaunchKernelGGL(window_rank_kernel<16>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
+                         colIdx, N, range, nPasses, blockPartition, edgeToColumn, edgeToRow, hdr);
+    else
+      hipLaunchKernelGGL(window_rank_kernel<8>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
+                         colIdx, N, range, nPasses, blockPartition, edgeToColumn, edgeToRow, hdr);
+    F3S_HIP_CHECK(hipGetLastError());
+  }
+  hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
+                     nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
+  F3S_HIP_CHECK(hipGetLastError());
+  WsHeader host;
+  F3S_HIP_CHECK(hipMemcpyAsync(&host, hdr, sizeof(WsHeader), hipMemcpyDeviceToHost, stream));
+  F3S_HIP_CHECK(hipStreamSynchronize(stream));
+  if (host.error) return fail(-4, "f3s_preprocess_count: column index outside [0, %d)", N);
+  *nTcbHost = host.nTcb;
+  return 0;
+}
+
+int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                           int W, const int32_t* edgeToColumn, const int32_t* rowWindowOffset,
+                           int64_t nTcb, int32_t* tcblockRowid, uint8_t* tcblocktileId,
+                           int32_t* tcblockOffset, int32_t* sparseAToXidx, uint64_t* bitmap,
+                           hipStream_t stream) {
+  if (H != 16 || (W != 16 && W != 8))
+    return fail(-2, "f3s_preprocess_fill: block %dx%d unsupported (16x16 or 16x8)", H, W);
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  if (nRW == 0) {
+    hipLaunchKernelGGL(set_tail_kernel, dim3(1), dim3(1), 0, stream, tcblockOffset,
+                       (long long)nTcb, E);
+    F3S_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
+  auto bm = reinterpret_cast<unsigned long long*>(bitmap);
+  if (W == 16)
+    hipLaunchKernelGGL(window_fill_kernel<16>, dim3(nRW), dim3(kBlock), 0, stream, rowPtr, colIdx,
+                       N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid,
+                       tcblocktileId, tcblockOffset, sparseAToXidx, bm);
+  else
+    hipLaunchKernelGGL(window_fill_kernel<8>, dim3(nRW), dim3(kBlock), 0, stream, rowPtr, colIdx,
+                       N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid,
+                       tcblocktileId, tcblockOffset, sparseAToXidx, bm);
+  F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+}  // namespace f3s

@@ -1,0 +1,115 @@
+/*
+ * f3s_amd.h -- C ABI of the MI355X (gfx950) Fused3S library, libf3s_amd.so.
+ *
+ * Plain pointers and sizes only. Unless stated otherwise every pointer is DEVICE memory on the
+ * current HIP device, int32 arrays are 4-byte aligned, sparseAToXidx / Q / K / V / out are
+ * 16-byte aligned, and `stream` is a hipStream_t passed as void* (NULL = default stream).
+ * Every entry point returns 0 on success and a negative code on failure; the message is then
+ * available from f3s_last_error() (per thread). Nothing here calls exit(): the reference's
+ * printf + exit(-1) error path (src/utils.cu:72-77, src/F3S_kernel.cu:662-666) becomes a status.
+ *
+ * Citations are to the HPCForge/Fused3S sources each entry point replaces.
+ */
+#ifndef F3S_AMD_H
+#define F3S_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define F3S_DTYPE_F16 0
+#define F3S_DTYPE_BF16 1
+
+/* ABI version of this header (bumped on incompatible change). */
+int f3s_abi_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). Never NULL. */
+const char* f3s_last_error(void);
+
+/*
+ * Bytes of device scratch f3s_preprocess_count needs for a graph of N nodes and E edges.
+ * Replaces the thrust::device_vector temporaries of seg_sort_dequ and
+ * sort_row_windows_by_tcb_count (src/utils.cu:281-284, 297-298, 404-405): the caller owns
+ * the allocation instead of the library.
+ */
+size_t f3s_preprocess_workspace_bytes(int N, int E);
+
+/*
+ * Phase 1 of F3S.preprocess_gpu (src/F3S.cpp:40-87): everything whose size is known up front.
+ * Replaces fill_edgeToRow_cuda (src/utils.cu:343-368, with edgeToRow[e] = row(e) for every
+ * edge -- the reference's grid-stride slip at :348 is not reproduced), fill_segment_cuda +
+ * thrust::sort + generate_edgetocolumn_cuda (src/utils.cu:371-396, 281-292, 131-170), the
+ * inclusive scan into rowWindowOffset (src/utils.cu:293-300) and
+ * sort_row_windows_by_tcb_count (src/utils.cu:400-436; equal counts keep ascending window id).
+ *
+ *   rowPtr  [N+1], colIdx [E]      CSR, int32; columns of a row may be unsorted or repeated
+ *   H, W                           TC-block height (16) and width (16, or 8 for the 16x8 layout)
+ *   blockPartition   [ceil(N/H)]   out: TC blocks per row window
+ *   edgeToColumn     [E]           out: rank of the edge's column among the window's sorted
+ *                                  unique columns
+ *   edgeToRow        [E]           out: row of each edge
+ *   rowWindowOffset  [ceil(N/H)+1] out: exclusive prefix of blockPartition
+ *   sortedRowWindows [ceil(N/H)]   out: windows by descending TC-block count
+ *   workspace, ws_bytes            device scratch of f3s_preprocess_workspace_bytes(N, E)
+ *   nTCB_host                      HOST pointer, out: total TC blocks (the reference's D->H
+ *                                  copy at src/utils.cu:307-309); the call synchronises `stream`
+ * Outputs are fully written; they need not be zeroed by the caller.
+ */
+int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                         int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                         int32_t* rowWindowOffset, int32_t* sortedRowWindows, void* workspace,
+                         size_t ws_bytes, int64_t* nTCB_host, void* stream);
+
+/*
+ * Phase 2 of F3S.preprocess_gpu: the outputs sized by nTCB. Replaces
+ * generate_tcblock_rowid_cuda (src/utils.cu:53-78), generate_tcoffset_id_atob_cuda with
+ * update_bitmap (src/utils.cu:23-36, 173-267) and the inclusive scan into tcblock_offset
+ * (src/utils.cu:333-337). No limit on TC blocks per window (the reference exits above
+ * 25 599, src/utils.cu:235-239).
+ *
+ *   edgeToColumn, rowWindowOffset  as produced by f3s_preprocess_count
+ *   tcblockRowid   [nTCB]          out: row window of each TC block
+ *   tcblocktileId  [E]  (uint8)    out: row_local*W + col_local, grouped by TC block, CSR order
+ *   tcblockOffset  [nTCB+1]        out: exclusive prefix of per-block nnz
+ *   sparseAToXidx  [nTCB*W]        out: original column of each compacted slot, 0 when unused
+ *   tcbBitMap      [nTCB*H*W/64] (uint64)  out: 8x8 sub-blocks in column-major order,
+ *                                  row-major and MSB-first inside a sub-block
+ * Asynchronous on `stream`. Outputs are fully written.
+ */
+int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                        const int32_t* edgeToColumn, const int32_t* rowWindowOffset, int64_t nTCB,
+                        int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                        int32_t* sparseAToXidx, uint64_t* tcbBitMap, void* stream);
+
+/*
+ * Fused SDDMM -> softmax -> SpMM over 16x16 TC blocks. Replaces f3sCuda1tb1rw,
+ * f3sCuda1tb1rwScheduled (src/F3S_kernel.cu:393-458, 581-671) and the kernels they launch
+ * (f3sKernel1tb1rw :997-1175, f3sKernel1tb1rwScheduled :1999-2182,
+ * f3sKernel1tb1rwScheduledPermutedQKV[ScaleQK] :1371-1800, f2sKernel1tb1rw :2186-2327).
+ *
+ *   rowWindowOffset [nRW+1], sparseAToXidx [nTCB*16], tcbBitMap [nTCB*4]   from preprocessing
+ *   windowOrder [nRW] or NULL      launch order of the row windows: sortedRowWindows for the
+ *                                  heavy-first schedule, NULL for natural order
+ *   N, d                           nodes; head dimension (32, 64 or 128)
+ *   dtype                          F3S_DTYPE_F16 (the reference's only type)
+ *   Q, K, V [N*d]                  row-major, contiguous
+ *   scalingFactor                  unmasked scores are DIVIDED by it (src/F3S_kernel.cu:1666-1667);
+ *                                  1.0 = unscaled (:612-613)
+ *   applySoftmax                   0 = SDDMM -> SpMM only (src/F3S_kernel.cu:420-443)
+ *   out [N*d] float                fully written (rows without edges get 0)
+ *   cuTimer                        NULL, or 3*nRW uint64 {begin, end, cu id} per workgroup
+ *                                  (the Clocked variants, src/F3S_kernel.cu:1178-1368, 1803-1997)
+ * Asynchronous on `stream`.
+ */
+int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int d,
+                      int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
+                      int applySoftmax, float* out, unsigned long long* cuTimer, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* F3S_AMD_H */

@@ -1,0 +1,501 @@
+/*
+ * f3s_oracle.c -- CPU restatement of the Fused3S hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker, never the product: only tests/, the smoke check and the
+ * benchmark's cpu_baseline leg may load it.  The shipped library (fused3s_amd/csrc) must
+ * never link, call or fall back to anything in here.
+ *
+ * Every function states the reference lines it follows (paths relative to the
+ * HPCForge/Fused3S checkout).  The reference itself is CUDA-only (inline PTX mma.sync,
+ * Thrust-on-CUDA), so it cannot be compiled here; this restatement is pinned instead by
+ * hand-derived known-answer vectors, by an independent dense-matrix derivation and by
+ * closed-form special cases (tests/test_oracle_*.py).
+ *
+ * Pinning status
+ *   preprocess_count / preprocess_fill : pinned (hand KATs + dense brute force + invariants),
+ *       except sortedRowWindows tie order, which the reference leaves to thrust::sort_by_key
+ *       (radix path => stable in practice, not promised by the API): parity unpinned for ties.
+ *   attention_textbook                 : pinned (dense fp64 masked softmax, closed forms).
+ *   attention_ref (reference numerics) : pinned to the textbook within the stated tolerance;
+ *       its bit-level behaviour (tensor-core summation order, __expf, __frcp_rn under
+ *       -use_fast_math) could only be pinned by a CUDA run: parity unpinned at bit level.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------ helpers */
+
+static int cmp_i32(const void *a, const void *b) {
+  int32_t x = *(const int32_t *)a, y = *(const int32_t *)b;
+  return (x > y) - (x < y);
+}
+
+static inline int imin(int a, int b) { return a < b ? a : b; }
+
+/* IEEE binary16 -> binary32, exact. */
+static float half_bits_to_float(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  uint32_t out;
+  if (exp == 0) {
+    if (man == 0) {
+      out = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do {
+        man <<= 1;
+        e++;
+      } while ((man & 0x400u) == 0);
+      man &= 0x3ffu;
+      out = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+    }
+  } else if (exp == 31) {
+    out = sign | 0x7f800000u | (man << 13);
+  } else {
+    out = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &out, 4);
+  return f;
+}
+
+/* binary32 -> binary16 with round-to-nearest-even (what __float2half does,
+ * F3S_kernel.cu:938-945). Returns the rounded value as a float. */
+static float round_to_half(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint32_t sign = x & 0x80000000u;
+  uint32_t ax = x & 0x7fffffffu;
+  uint16_t h;
+  if (ax >= 0x7f800000u) { /* inf / nan */
+    h = (uint16_t)(0x7c00u | ((ax > 0x7f800000u) ? 0x200u : 0));
+  } else if (ax >= 0x477ff000u) { /* rounds to >= 65520 -> inf */
+    h = 0x7c00u;
+  } else if (ax < 0x33000001u) { /* < 2^-25 (or == 2^-25, ties to even 0) */
+    h = 0;
+  } else {
+    int e = (int)(ax >> 23) - 127;
+    uint32_t m = (ax & 0x7fffffu) | 0x800000u;
+    int shift;
+    uint32_t base;
+    if (e < -14) { /* subnormal half */
+      shift = 13 + (-14 - e);
+      base = 0;
+    } else {
+      shift = 13;
+      base = (uint32_t)(e + 15) << 10;
+      m &= 0x7fffffu;
+    }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) q++;
+    h = (uint16_t)(base + q); /* carry into the exponent is correct by construction */
+  }
+  h |= (uint16_t)(sign >> 16);
+  return half_bits_to_float(h);
+}
+
+static float bf16_bits_to_float(uint16_t b) {
+  uint32_t x = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+static float *to_float(const uint16_t *src, int64_t n, int dtype) {
+  float *dst = (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+  if (!dst) return NULL;
+  if (dtype == 0) {
+    for (int64_t i = 0; i < n; i++) dst[i] = half_bits_to_float(src[i]);
+  } else {
+    for (int64_t i = 0; i < n; i++) dst[i] = bf16_bits_to_float(src[i]);
+  }
+  return dst;
+}
+
+/* exported so tests can pin the conversions against numpy.float16 */
+float f3s_oracle_half_to_float(uint16_t h) { return half_bits_to_float(h); }
+float f3s_oracle_round_to_half(float f) { return round_to_half(f); }
+
+/* ------------------------------------------------------------ preprocessing */
+
+/*
+ * Phase 1: per 16-row window, the ascending unique column ids U_w, the TC-block count
+ * ceil(|U_w|/W), and the compacted column rank of every edge.
+ *   generate_edgetocolumn       src/utils.cu:131-153  (window bounds :137-140, early
+ *                               return for empty windows :141-142, count :146-148,
+ *                               rank by binary search :149-152)
+ *   inplace_deduplication       src/utils.cu:120-130
+ *   sorted (window,col) input   src/utils.cu:281-289 (thrust::sort on the zipped pair)
+ *   rowWindowOffset             src/utils.cu:293-300 (inclusive scan into offset+1)
+ * blockPartition entries of empty windows are left as the caller passed them (zeros in
+ * every reference call site), exactly as the reference leaves them.
+ * Returns the TC-block total (reference: atomicAdd into blocknum, :147).
+ */
+int64_t f3s_oracle_preprocess_count(const int32_t *rowPtr, const int32_t *colIdx, int N, int H,
+                                    int W, int32_t *blockPartition, int32_t *edgeToColumn,
+                                    int32_t *rowWindowOffset) {
+  int nRW = (N + H - 1) / H;
+  int64_t total = 0;
+  int32_t *tmp = NULL;
+  int64_t cap = 0;
+  for (int w = 0; w < nRW; w++) {
+    int64_t s = rowPtr[(int64_t)w * H];
+    int64_t e = rowPtr[imin(w * H + H, N)];
+    int64_t n = e - s;
+    if (n == 0) continue;
+    if (n > cap) {
+      free(tmp);
+      cap = n * 2;
+      tmp = (int32_t *)malloc(sizeof(int32_t) * (size_t)cap);
+      if (!tmp) return -1;
+    }
+    memcpy(tmp, colIdx + s, sizeof(int32_t) * (size_t)n);
+    qsort(tmp, (size_t)n, sizeof(int32_t), cmp_i32);
+    int64_t loc = 0; /* index of the last unique element, as in inplace_deduplication */
+    for (int64_t cur = 1; cur < n; cur++) {
+      if (tmp[cur] != tmp[cur - 1]) tmp[++loc] = tmp[cur];
+    }
+    int num = (int)((loc + W) / W);
+    blockPartition[w] = num;
+    total += num;
+    for (int64_t k = s; k < e; k++) {
+      int32_t target = colIdx[k];
+      int64_t lo = 0, hi = loc;
+      int64_t idx = -1;
+      while (lo <= hi) {
+        int64_t mid = lo + (hi - lo) / 2;
+        if (tmp[mid] == target) {
+          idx = mid;
+          break;
+        }
+        if (tmp[mid] < target)
+          lo = mid + 1;
+        else
+          hi = mid - 1;
+      }
+      edgeToColumn[k] = (int32_t)idx;
+    }
+  }
+  free(tmp);
+  rowWindowOffset[0] = 0;
+  for (int w = 0; w < nRW; w++) rowWindowOffset[w + 1] = rowWindowOffset[w] + blockPartition[w];
+  return total;
+}
+
+/*
+ * edgeToRow.  Intent of fill_edgeToRow (src/utils.cu:343-352): edgeToRow[e] = row(e).
+ * The reference's inner loop strides by gridDim.x instead of blockDim.x; with
+ * G = min(ceil(N/32), 10000) blocks (:354-360) an edge at in-row offset k is only written
+ * when k = tx + j*G for some lane tx in [0,32), everything else keeps the caller's value
+ * (zero at every call site).  emulate_stride_bug != 0 reproduces that literally;
+ * emulate_stride_bug == 0 is the evident intent and what the reference produces whenever
+ * G <= 32 (N <= 1024, the size of its own accuracy test).
+ * The caller passes edgeToRow zero-filled when emulating.
+ */
+void f3s_oracle_fill_edge_to_row(const int32_t *rowPtr, int N, int emulate_stride_bug,
+                                 int32_t *edgeToRow) {
+  if (!emulate_stride_bug) {
+    for (int r = 0; r < N; r++)
+      for (int64_t k = rowPtr[r]; k < rowPtr[r + 1]; k++) edgeToRow[k] = r;
+    return;
+  }
+  int64_t G = ((int64_t)N + 31) / 32;
+  if (G > 10000) G = 10000;
+  if (G < 1) G = 1;
+  for (int r = 0; r < N; r++)
+    for (int tx = 0; tx < 32; tx++)
+      for (int64_t k = (int64_t)rowPtr[r] + tx; k < rowPtr[r + 1]; k += G) edgeToRow[k] = r;
+}
+
+typedef struct {
+  int32_t count;
+  int32_t id;
+} win_key_t;
+
+static int cmp_win_desc_stable(const void *a, const void *b) {
+  const win_key_t *x = (const win_key_t *)a, *y = (const win_key_t *)b;
+  if (x->count != y->count) return (x->count < y->count) - (x->count > y->count); /* desc */
+  return (x->id > y->id) - (x->id < y->id); /* ties: ascending window id */
+}
+
+/*
+ * Phase 2: everything whose size depends on the TC-block total.
+ *   generate_tcoffset_id_atob   src/utils.cu:173-224 (per-TCB nnz :200-206, exclusive
+ *                               positions :209-211, tile ids :218-219, bitmap :220,
+ *                               sparseAToXidx :221)
+ *   update_bitmap               src/utils.cu:23-36 -- called with (blockSize_w, blockSize_h)
+ *                               in swapped positions (:220), so the sub-block index is
+ *                               (col_local/8)*(W/8) + row_local/8
+ *   tcblock_offset              src/utils.cu:318,331,333-337 (nnz written at offset+1, then an
+ *                               inclusive scan over nTCB+1 entries)
+ *   generate_tcblock_rowid      src/utils.cu:53-65
+ *   sort_row_windows_by_tcb_count  src/utils.cu:400-436 (descending TC-block count; ties in
+ *                               ascending window id = stable, see the header)
+ * Outputs are fully written here (the reference gets its zeros from torch::zeros,
+ * src/utils.cu:310-324).
+ */
+void f3s_oracle_preprocess_fill(const int32_t *rowPtr, const int32_t *colIdx, int N, int H, int W,
+                                const int32_t *edgeToColumn, const int32_t *edgeToRow,
+                                const int32_t *rowWindowOffset, int32_t *tcblockRowid,
+                                uint8_t *tcblocktileId, int32_t *tcblockOffset,
+                                int32_t *sparseAToXidx, uint64_t *bitmap,
+                                int32_t *sortedRowWindows) {
+  int nRW = (N + H - 1) / H;
+  int64_t nTCB = rowWindowOffset[nRW];
+  int wordsPerTcb = H * W / 64;
+  int64_t E = rowPtr[N];
+  memset(sparseAToXidx, 0, sizeof(int32_t) * (size_t)(nTCB * W));
+  memset(bitmap, 0, sizeof(uint64_t) * (size_t)(nTCB * wordsPerTcb));
+  memset(tcblockOffset, 0, sizeof(int32_t) * (size_t)(nTCB + 1));
+  memset(tcblocktileId, 0, (size_t)E);
+  for (int w = 0; w < nRW; w++) {
+    int64_t base = rowWindowOffset[w];
+    int64_t nb = rowWindowOffset[w + 1] - base;
+    for (int64_t t = 0; t < nb; t++) tcblockRowid[base + t] = w;
+    if (nb == 0) continue;
+    int64_t s = rowPtr[(int64_t)w * H];
+    int64_t e = rowPtr[imin(w * H + H, N)];
+    if (e == s) continue;
+    int32_t *nnz = (int32_t *)calloc((size_t)nb, sizeof(int32_t));
+    int32_t *start = (int32_t *)calloc((size_t)nb, sizeof(int32_t));
+    int32_t *pos = (int32_t *)calloc((size_t)nb, sizeof(int32_t));
+    for (int64_t k = s; k < e; k++) nnz[edgeToColumn[k] / W]++;
+    for (int64_t t = 0; t < nb; t++) tcblockOffset[1 + base + t] = nnz[t];
+    for (int64_t t = 1; t < nb; t++) start[t] = start[t - 1] + nnz[t - 1];
+    for (int64_t k = s; k < e; k++) {
+      int col = edgeToColumn[k];
+      int t = col / W;
+      int rl = edgeToRow[k] % H;
+      int cl = col % W;
+      tcblocktileId[s + start[t] + pos[t]] = (uint8_t)(rl * W + cl);
+      int sub = (cl / 8) * (W / 8) + rl / 8;
+      int bit = (rl % 8) * 8 + cl % 8;
+      bitmap[(base + t) * wordsPerTcb + sub] |= 1ULL << (63 - bit);
+      sparseAToXidx[(base + t) * W + cl] = colIdx[k];
+      pos[t]++;
+    }
+    free(nnz);
+    free(start);
+    free(pos);
+  }
+  for (int64_t t = 1; t <= nTCB; t++) tcblockOffset[t] += tcblockOffset[t - 1];
+
+  win_key_t *keys = (win_key_t *)malloc(sizeof(win_key_t) * (size_t)(nRW > 0 ? nRW : 1));
+  for (int w = 0; w < nRW; w++) {
+    keys[w].count = rowWindowOffset[w + 1] - rowWindowOffset[w];
+    keys[w].id = w;
+  }
+  qsort(keys, (size_t)nRW, sizeof(win_key_t), cmp_win_desc_stable);
+  for (int w = 0; w < nRW; w++) sortedRowWindows[w] = keys[w].id;
+  free(keys);
+}
+
+/* ---------------------------------------------------------------- attention */
+
+/* Bit test as the kernels consume it: 16x16 TCB, src/F3S_kernel.cu:1447-1451. */
+static inline int tcb_bit(const uint64_t *bitmap, int64_t t, int rl, int cl) {
+  int sub = (cl / 8) * 2 + rl / 8;
+  int bit = (rl % 8) * 8 + cl % 8;
+  return (int)((bitmap[t * 4 + sub] >> (63 - bit)) & 1ULL);
+}
+
+/*
+ * Reference-emulating fused 3S over 16x16 TC blocks.
+ *   f3sKernel1tb1rwScheduledPermutedQKV[ScaleQK]   src/F3S_kernel.cu:1371-1800
+ *   launcher (padded output, slice to N)            src/F3S_kernel.cu:581-671
+ * Per window, chunks of C = nWarpPerBlock/2 consecutive TC blocks (:1414-1419):
+ *   S = Q K^T in fp32 from fp16 products (:1424-1446); masked entries become 0.0 (:1447-1451),
+ *   unmasked ones are divided by scalingFactor in the ScaleQK kernel (:1666-1667; the launcher
+ *   picks the unscaled kernel when scalingFactor == 1.0, :612-613);
+ *   running max starts at 0.0 and masked zeros take part in it (:1402-1406,1463-1490);
+ *   alpha = exp(m_old - m_new) (:1487-1490); E = (S == 0) ? 0 : exp(S - m_new) (:1492-1493);
+ *   row sum from un-rounded E with fma(alpha, l, sum) (:1495-1517);
+ *   P = fp16(E) (:938-945); O = alpha*O + P V in fp32 (:1519-1557);
+ *   out = O * (l == 0 ? 0 : 1/l) (:1560-1582).
+ * applySoftmax == 0 follows f2sKernel1tb1rw (src/F3S_kernel.cu:2186-2327): out = fp16(S) V with
+ * the same masking, no scaling.
+ * The window order is irrelevant to the result (windows are independent), so the
+ * sortedRowWindows argument of the reference is not needed here.
+ * Rows >= N of the last window are treated as all-zero Q and never written.
+ * dtype: 0 = fp16 inputs (the reference), 1 = bf16 inputs (beyond the reference: same
+ * algorithm, P still rounded to fp16).
+ */
+int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *sparseAToXidx,
+                             const uint64_t *bitmap, int N, int d, int dtype, const uint16_t *Q,
+                             const uint16_t *K, const uint16_t *V, float scalingFactor,
+                             int nWarpPerBlock, int applySoftmax, int winBegin, int winEnd,
+                             float *out) {
+  int nRW = (N + 15) / 16;
+  if (winBegin < 0) winBegin = 0;
+  if (winEnd > nRW || winEnd < 0) winEnd = nRW;
+  int C = nWarpPerBlock / 2;
+  if (C < 1) return -1;
+  float *Qf = to_float(Q, (int64_t)N * d, dtype);
+  float *Kf = to_float(K, (int64_t)N * d, dtype);
+  float *Vf = to_float(V, (int64_t)N * d, dtype);
+  if (!Qf || !Kf || !Vf) return -2;
+  int scale = (scalingFactor != 1.0f);
+#pragma omp parallel
+  {
+    float *S = (float *)malloc(sizeof(float) * (size_t)(C * 16));
+    float *P = (float *)malloc(sizeof(float) * (size_t)(C * 16));
+    float *O = (float *)malloc(sizeof(float) * (size_t)d);
+#pragma omp for schedule(dynamic, 4)
+    for (int w = winBegin; w < winEnd; w++) {
+      int64_t t0 = rowWindowOffset[w], t1 = rowWindowOffset[w + 1];
+      for (int rl = 0; rl < 16; rl++) {
+        int64_t r = (int64_t)w * 16 + rl;
+        if (r >= N) break;
+        const float *q = Qf + r * d;
+        float m = 0.0f, l = 0.0f;
+        for (int c = 0; c < d; c++) O[c] = 0.0f;
+        for (int64_t tc = t0; tc < t1; tc += C) {
+          int nb = (int)((t1 - tc) < C ? (t1 - tc) : C);
+          float mnew = m;
+          for (int b = 0; b < nb; b++) {
+            for (int j = 0; j < 16; j++) {
+              float s = 0.0f;
+              if (tcb_bit(bitmap, tc + b, rl, j)) {
+                const float *k = Kf + (int64_t)sparseAToXidx[(tc + b) * 16 + j] * d;
+                double acc = 0.0;
+                for (int c = 0; c < d; c++) acc += (double)q[c] * (double)k[c];
+                s = (float)acc;
+                if (applySoftmax && scale) s = s / scalingFactor;
+              }
+              S[b * 16 + j] = s;
+              if (s > mnew) mnew = s;
+            }
+          }
+          if (applySoftmax) {
+            float alpha = expf(m - mnew);
+            m = mnew;
+            float sum = 0.0f;
+            for (int i = 0; i < nb * 16; i++) {
+              float ev = (S[i] == 0.0f) ? 0.0f : expf(S[i] - mnew);
+              sum += ev;
+              P[i] = round_to_half(ev);
+            }
+            l = fmaf(alpha, l, sum);
+            for (int c = 0; c < d; c++) O[c] *= alpha;
+          } else {
+            for (int i = 0; i < nb * 16; i++) P[i] = round_to_half(S[i]);
+          }
+          for (int b = 0; b < nb; b++) {
+            for (int j = 0; j < 16; j++) {
+              float p = P[b * 16 + j];
+              if (p == 0.0f) continue;
+              const float *v = Vf + (int64_t)sparseAToXidx[(tc + b) * 16 + j] * d;
+              for (int c = 0; c < d; c++) O[c] += p * v[c];
+            }
+          }
+        }
+        float inv = 1.0f;
+        if (applySoftmax) inv = (l == 0.0f) ? 0.0f : 1.0f / l;
+        float *o = out + r * d;
+        for (int c = 0; c < d; c++) o[c] = O[c] * inv;
+      }
+    }
+    free(S);
+    free(P);
+    free(O);
+  }
+  free(Qf);
+  free(Kf);
+  free(Vf);
+  return 0;
+}
+
+/*
+ * Textbook masked-softmax attention straight from CSR, fp64 accumulation:
+ *   out[i,:] = sum_{j in N(i)} softmax_j(Q_i.K_j / scalingFactor) V_j ,
+ * N(i) = DISTINCT columns of CSR row i, empty row => 0.
+ *   row_wise_softmax_mask followed by S @ V   scripts/tests/test_f3s_accuracy.py:81-94,148-164
+ *   edge-wise SDDMM / segment softmax / SpMM  scripts/baseline_comp/baseline_comp_kernel_only.py:667-686
+ * Rows [rowBegin,rowEnd) only, so a bounded sample of a large graph can be checked or timed.
+ */
+int f3s_oracle_attention_textbook(const int32_t *rowPtr, const int32_t *colIdx, int N, int d,
+                                  int dtype, const uint16_t *Q, const uint16_t *K,
+                                  const uint16_t *V, float scalingFactor, int rowBegin,
+                                  int rowEnd, float *out) {
+  if (rowBegin < 0) rowBegin = 0;
+  if (rowEnd > N || rowEnd < 0) rowEnd = N;
+  float *Qf = to_float(Q, (int64_t)N * d, dtype);
+  float *Kf = to_float(K, (int64_t)N * d, dtype);
+  float *Vf = to_float(V, (int64_t)N * d, dtype);
+  if (!Qf || !Kf || !Vf) return -2;
+  int status = 0;
+#pragma omp parallel
+  {
+    int64_t cap = 64;
+    int32_t *cols = (int32_t *)malloc(sizeof(int32_t) * (size_t)cap);
+    double *sc = (double *)malloc(sizeof(double) * (size_t)cap);
+    double *acc = (double *)malloc(sizeof(double) * (size_t)d);
+#pragma omp for schedule(dynamic, 16)
+    for (int r = rowBegin; r < rowEnd; r++) {
+      int64_t s = rowPtr[r], e = rowPtr[r + 1];
+      int64_t n = e - s;
+      float *o = out + (int64_t)r * d;
+      if (n == 0) {
+        for (int c = 0; c < d; c++) o[c] = 0.0f;
+        continue;
+      }
+      if (n > cap) {
+        cap = n * 2;
+        cols = (int32_t *)realloc(cols, sizeof(int32_t) * (size_t)cap);
+        sc = (double *)realloc(sc, sizeof(double) * (size_t)cap);
+        if (!cols || !sc) {
+          status = -2;
+          continue;
+        }
+      }
+      memcpy(cols, colIdx + s, sizeof(int32_t) * (size_t)n);
+      qsort(cols, (size_t)n, sizeof(int32_t), cmp_i32);
+      int64_t u = 1;
+      for (int64_t i = 1; i < n; i++)
+        if (cols[i] != cols[u - 1]) cols[u++] = cols[i];
+      const float *q = Qf + (int64_t)r * d;
+      double mx = -INFINITY;
+      for (int64_t i = 0; i < u; i++) {
+        const float *k = Kf + (int64_t)cols[i] * d;
+        double a = 0.0;
+        for (int c = 0; c < d; c++) a += (double)q[c] * (double)k[c];
+        a /= (double)scalingFactor;
+        sc[i] = a;
+        if (a > mx) mx = a;
+      }
+      double den = 0.0;
+      for (int c = 0; c < d; c++) acc[c] = 0.0;
+      for (int64_t i = 0; i < u; i++) {
+        double p = exp(sc[i] - mx);
+        den += p;
+        const float *v = Vf + (int64_t)cols[i] * d;
+        for (int c = 0; c < d; c++) acc[c] += p * (double)v[c];
+      }
+      for (int c = 0; c < d; c++) o[c] = (float)(acc[c] / den);
+    }
+    free(cols);
+    free(sc);
+    free(acc);
+  }
+  free(Qf);
+  free(Kf);
+  free(Vf);
+  return status;
+}
+
+int f3s_oracle_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

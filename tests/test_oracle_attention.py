@@ -1,0 +1,160 @@
+"""Pins the attention oracles: the textbook one against a dense fp64 masked softmax and closed
+forms, the reference-emulating one against the textbook within the stated tolerance plus the
+reference's documented quirks."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import random_csr
+from ref_checks import dense_attention, dense_from_csr
+
+MAX_ABS = 2e-2   # tolerance of the attention output (fp16 in, fp32 accumulate)
+MEAN_REL = 1e-3
+
+
+def mean_rel(a, b):
+    return float(np.abs(a - b).mean() / max(np.abs(b).mean(), 1e-30))
+
+
+def feats(rng, N, d, std=1.0):
+    return [(rng.standard_normal((N, d)) * std).astype(np.float16) for _ in range(3)]
+
+
+def test_half_conversions_match_numpy(oracle_mod):
+    L = oracle_mod.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([L.f3s_oracle_half_to_float(int(b)) for b in bits], np.float32)
+    ok = (got == want) | (np.isnan(got) & np.isnan(want))
+    assert ok.all()
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32),
+        (rng.standard_normal(5000) * 1e-6).astype(np.float32),
+        (rng.standard_normal(2000) * 3e4).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, 2.0 ** -24, 2.0 ** -25,
+                  2.0 ** -25 * 1.0001, 2.0 ** -14, 1.00048828125, 1.0009765625 + 2.0 ** -12],
+                 np.float32)])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).astype(np.float32)
+    got = np.array([L.f3s_oracle_round_to_half(ctypes.c_float(float(x))) for x in xs], np.float32)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("seed,N,d,deg,dup,unsorted", [
+    (0, 40, 32, 5, False, False), (1, 97, 64, 12, True, True), (2, 150, 128, 3, False, True)])
+def test_textbook_matches_dense_fp64(oracle_mod, seed, N, d, deg, dup, unsorted):
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, dup=dup, unsorted=unsorted, empty_frac=0.1)
+    Q, K, V = feats(rng, N, d)
+    scale = float(np.sqrt(d))
+    got = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, scale)
+    want = dense_attention(rowPtr, colIdx, N, Q, K, V, scale)
+    assert np.abs(got - want).max() < 1e-5
+
+
+def test_closed_forms(oracle_mod):
+    rng = np.random.default_rng(7)
+    N, d = 48, 64
+    Q, K, V = feats(rng, N, d)
+    # degree-1 rows copy one V row; row 5 is empty; rows 40.. see identical keys -> plain mean
+    rows = []
+    for r in range(N):
+        if r == 5:
+            rows.append([])
+        elif r < 40:
+            rows.append([(7 * r + 3) % N])
+        else:
+            rows.append([1, 2, 3, 4])
+    K[2] = K[1]
+    K[3] = K[1]
+    K[4] = K[1]
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum([len(x) for x in rows])
+    colIdx = np.array([c for x in rows for c in x], np.int32)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    for out in (oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, 8.0),
+                oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                         pre["tcbBitMap"], N, Q, K, V, 8.0)):
+        for r in range(40):
+            if r == 5:
+                assert np.all(out[r] == 0)
+            else:
+                assert np.abs(out[r] - V[(7 * r + 3) % N].astype(np.float32)).max() < 2e-3
+        mean = V[1:5].astype(np.float64).mean(axis=0)
+        for r in range(40, N):
+            assert np.abs(out[r] - mean).max() < 2e-3
+
+
+@pytest.mark.parametrize("nwarp", [2, 8, 16])
+@pytest.mark.parametrize("seed,N,d,deg", [(0, 300, 64, 25), (1, 1000, 128, 100), (2, 77, 32, 6)])
+def test_reference_numerics_agree_with_textbook_within_tolerance(oracle_mod, seed, N, d, deg, nwarp):
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, hub=13)
+    Q, K, V = feats(rng, N, d)
+    scale = float(np.sqrt(d))
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    ref = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                   N, Q, K, V, scale, nWarpPerBlock=nwarp)
+    txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, scale)
+    assert np.abs(ref - txt).max() < MAX_ABS
+    assert mean_rel(ref, txt) < MEAN_REL
+
+
+def test_reference_accuracy_harness_shape(oracle_mod):
+    """The reference's own check (scripts/tests/test_f3s_accuracy.py:96-236): 1000 nodes, 10 %
+    dense mask, d=128, uniform [0,1) features, no scaling; it prints the relative Frobenius
+    error and expects it to be small."""
+    rng = np.random.default_rng(0)
+    N, d = 1000, 128
+    A = rng.random((N, N)) < 0.1
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(A.sum(axis=1))
+    colIdx = np.nonzero(A)[1].astype(np.int32)
+    Q, K, V = [rng.random((N, d)).astype(np.float16) for _ in range(3)]
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    ref = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                   N, Q, K, V, 1.0)
+    want = dense_attention(rowPtr, colIdx, N, Q, K, V, 1.0)
+    rel_fro = np.linalg.norm(ref - want) / np.linalg.norm(want)
+    assert rel_fro < 2e-3
+
+
+def test_reference_quirks(oracle_mod):
+    rng = np.random.default_rng(3)
+    N, d = 32, 64
+    Q, K, V = feats(rng, N, d)
+    rowPtr, colIdx = random_csr(rng, N, 6)
+    Q[3] = 0  # every score of row 3 is exactly 0.0 -> treated as masked -> l == 0 -> output 0
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    args = (pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"], N, Q, K, V)
+    ref = oracle_mod.attention_ref(*args, 8.0)
+    txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, 8.0)
+    if rowPtr[4] > rowPtr[3]:
+        assert np.all(ref[3] == 0) and np.abs(txt[3]).max() > 0
+    others = [r for r in range(N) if r != 3]
+    assert np.abs(ref[others] - txt[others]).max() < MAX_ABS
+    # running max starts at 0: scores far below zero underflow in fp16 and are lost
+    Qn = Q.copy()
+    Qn[7] = 60.0
+    Kn = K.copy()
+    Kn[:] = -1.0
+    low = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                   N, Qn, Kn, V, 1.0)
+    if rowPtr[8] > rowPtr[7]:
+        assert np.all(low[7] == 0)  # exp(-3840) == 0
+
+
+def test_sddmm_spmm_without_softmax(oracle_mod):
+    rng = np.random.default_rng(5)
+    N, d = 90, 64
+    rowPtr, colIdx = random_csr(rng, N, 8)
+    Q, K, V = feats(rng, N, d, std=0.5)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    got = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                   N, Q, K, V, 1.0, applySoftmax=False)
+    A = dense_from_csr(rowPtr, colIdx, N) > 0
+    S = (Q.astype(np.float64) @ K.astype(np.float64).T) * A
+    want = S.astype(np.float16).astype(np.float64) @ V.astype(np.float64)
+    assert np.abs(got - want).max() < 5e-3 * max(1.0, np.abs(want).max())
