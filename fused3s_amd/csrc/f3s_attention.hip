@@ -62,7 +62,7 @@ template <int D, int NWAVES, bool SOFTMAX>
 __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
-    const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+    int nRW, const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     const _Float16* __restrict__ V, float scaleLog2, float* __restrict__ out) {
   constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
   constexpr int KS = D / 32;  // MFMA k-steps of the score product
@@ -71,9 +71,10 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
 
   __shared__ float sM[NWAVES][16];
   __shared__ float sL[NWAVES][16];
-  __shared__ float sO[NWAVES][16][OSTRIDE];
+  __shared__ __align__(16) float sO[NWAVES][16][OSTRIDE];
 
   const int w = windowOrder ? windowOrder[blockIdx.x] : (int)blockIdx.x;
+  if ((unsigned)w >= (unsigned)nRW) return;  // a corrupt order entry must not index out of range
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int g = lane >> 4;
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
     const int tB = hasB ? tA + 1 : tA;
 
     // gathered K rows -> A operand
-    const int kRowA = sparseAToXidx[tA * 16 + c];
-    const int kRowB = sparseAToXidx[tB * 16 + c];
+    const int kRowA = sparseAToXidx[(int64_t)tA * 16 + c];
+    const int kRowB = sparseAToXidx[(int64_t)tB * 16 + c];
     const half8* kpA = reinterpret_cast<const half8*>(K + (int64_t)kRowA * D) + g;
     const half8* kpB = reinterpret_cast<const half8*>(K + (int64_t)kRowB * D) + g;
     half8 kA[KS], kB[KS];
@@ -123,8 +124,8 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
       kB[i] = kpB[4 * i];
     }
     // V rows of this lane's 8 contraction slots
-    const int4 vIdxA = reinterpret_cast<const int4*>(sparseAToXidx + tA * 16)[g];
-    const int4 vIdxB = reinterpret_cast<const int4*>(sparseAToXidx + tB * 16)[g];
+    const int4 vIdxA = reinterpret_cast<const int4*>(sparseAToXidx + (int64_t)tA * 16)[g];
+    const int4 vIdxB = reinterpret_cast<const int4*>(sparseAToXidx + (int64_t)tB * 16)[g];
     const int vr[8] = {vIdxA.x, vIdxA.y, vIdxA.z, vIdxA.w, vIdxB.x, vIdxB.y, vIdxB.z, vIdxB.w};
     vrow_t vv[8];
 #pragma unroll
@@ -244,7 +245,7 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
   const int nRW = (N + kWinRows - 1) / kWinRows;
   if (nRW == 0) return 0;
   hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX>), dim3(nRW), dim3(NWAVES * 64), 0, stream,
-                     rwo, order, atox, reinterpret_cast<const uint8_t*>(bitmap), N,
+                     rwo, order, atox, reinterpret_cast<const uint8_t*>(bitmap), N, nRW,
                      static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
                      static_cast<const _Float16*>(V), scaleLog2, out);
   F3S_HIP_CHECK(hipGetLastError());

@@ -1,0 +1,132 @@
+"""Fused 3S attention (HIP, through the C ABI) against the CPU oracles.
+
+Tolerance (fp16 inputs, fp32 accumulation): max-abs 2e-2 and mean-relative 1e-3 against the
+reference-emulating oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+
+pytestmark = pytest.mark.gpu
+MAX_ABS = 2e-2
+MEAN_REL = 1e-3
+
+
+def mean_rel(a, b):
+    return float(np.abs(a - b).mean() / max(np.abs(b).mean(), 1e-30))
+
+
+def gpu_attention(pre, N, Q, K, V, scale, order=None, softmax=True):
+    from fused3s_amd import capi
+    dev = "cuda"
+    rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
+    atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
+    bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
+    od = None if order is None else torch.as_tensor(np.asarray(order, np.int32)).to(dev)
+    out = capi.attention(rwo, od, atox, bm, N, torch.as_tensor(Q).to(dev),
+                         torch.as_tensor(K).to(dev), torch.as_tensor(V).to(dev), scale, softmax)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def feats(rng, N, d, std=1.0):
+    return [(rng.standard_normal((N, d)) * std).astype(np.float16) for _ in range(3)]
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("seed,N,deg,hub", [(0, 300, 25, 13), (1, 1000, 100, 0), (2, 77, 6, 0),
+                                            (3, 16, 2, 0), (4, 4099, 40, 100)])
+def test_matches_reference_numerics(oracle_mod, d, seed, N, deg, hub):
+    print("case d=%d seed=%d N=%d" % (d, seed, N), flush=True)
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, hub=hub, empty_frac=0.05)
+    Q, K, V = feats(rng, N, d)
+    scale = float(np.sqrt(d))
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, Q, K, V, scale)
+    txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, scale)
+    for order in (None, pre["sortedRowWindows"]):
+        got = gpu_attention(pre, N, Q, K, V, scale, order)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() < MAX_ABS
+        assert mean_rel(got, want) < MEAN_REL
+        assert np.abs(got - txt).max() < MAX_ABS
+
+
+def test_unscaled_uniform_features_like_reference_harness(oracle_mod):
+    """scripts/tests/test_f3s_accuracy.py:96-236: N=1000, 10 % dense, d=128, U[0,1), no scaling."""
+    print("case harness", flush=True)
+    rng = np.random.default_rng(0)
+    N, d = 1000, 128
+    A = rng.random((N, N)) < 0.1
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(A.sum(axis=1))
+    colIdx = np.nonzero(A)[1].astype(np.int32)
+    Q, K, V = [rng.random((N, d)).astype(np.float16) for _ in range(3)]
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, Q, K, V, 1.0)
+    got = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"])
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 2e-3
+    assert np.abs(got - want).max() < MAX_ABS
+
+
+def test_closed_forms_and_quirks(oracle_mod):
+    print("case closed_forms", flush=True)
+    rng = np.random.default_rng(7)
+    N, d = 48, 64
+    Q, K, V = feats(rng, N, d)
+    rows = []
+    for r in range(N):
+        rows.append([] if r == 5 else ([(7 * r + 3) % N] if r < 40 else [1, 2, 3, 4]))
+    K[2] = K[1]
+    K[3] = K[1]
+    K[4] = K[1]
+    Q[9] = 0  # all scores exactly zero: dropped like masked entries -> row sum 0 -> output 0
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum([len(x) for x in rows])
+    colIdx = np.array([c for x in rows for c in x], np.int32)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    out = gpu_attention(pre, N, Q, K, V, 8.0)
+    for r in range(40):
+        if r in (5, 9):
+            assert np.all(out[r] == 0)
+        else:
+            assert np.abs(out[r] - V[(7 * r + 3) % N].astype(np.float32)).max() < 2e-3
+    mean = V[1:5].astype(np.float64).mean(axis=0)
+    for r in range(40, N):
+        assert np.abs(out[r] - mean).max() < 2e-3
+
+
+def test_sddmm_spmm_without_softmax(oracle_mod):
+    print("case no_softmax", flush=True)
+    rng = np.random.default_rng(5)
+    N, d = 900, 64
+    rowPtr, colIdx = random_csr(rng, N, 20)
+    Q, K, V = feats(rng, N, d, std=0.5)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
+    got = gpu_attention(pre, N, Q, K, V, 1.0, None, softmax=False)
+    assert np.abs(got - want).max() < 2e-2 * max(1.0, np.abs(want).max())
+    assert mean_rel(got, want) < MEAN_REL
+
+
+def test_end_to_end_hip_preprocess_then_attention(oracle_mod):
+    """CSR -> HIP preprocessing -> HIP attention, checked against the textbook oracle."""
+    print("case end_to_end", flush=True)
+    from fused3s_amd import capi, synth
+    rp, ci = synth.make_graph("cfg1_gnm_2708")
+    N = rp.numel() - 1
+    Q, K, V = synth.features(N, 64, seed=0)
+    pre = capi.preprocess(rp.cuda(), ci.cuda(), N)
+    out = capi.attention(pre["rowWindowOffset"], pre["sortedRowWindows"], pre["sparseAToXidx"],
+                         pre["tcbBitMap"], N, Q.cuda(), K.cuda(), V.cuda(), 8.0)
+    torch.cuda.synchronize()
+    txt = oracle_mod.attention_textbook(rp.numpy(), ci.numpy(), N, Q.numpy(), K.numpy(),
+                                        V.numpy(), 8.0)
+    got = out.cpu().numpy()
+    assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL

@@ -1,0 +1,126 @@
+"""HIP preprocessing (through the C ABI) against the CPU oracle: bit-exact on every output."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+from ref_checks import compare_preprocess
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+KAT = json.load(open(os.path.join(HERE, "golden", "preprocess_kat.json")))["cases"]
+
+
+def to_host(res):
+    out = {}
+    for k, v in res.items():
+        if torch.is_tensor(v):
+            v = v.cpu()
+            out[k] = v.view(torch.int64).numpy().view(np.uint64) if v.dtype == torch.uint64 \
+                else v.numpy()
+        else:
+            out[k] = v
+    return out
+
+
+def run_gpu(rowPtr, colIdx, N, W=16):
+    from fused3s_amd import capi
+    rp = torch.as_tensor(np.asarray(rowPtr, np.int32)).cuda()
+    ci = torch.as_tensor(np.asarray(colIdx, np.int32)).cuda()
+    res = capi.preprocess(rp, ci, N, 16, W)
+    torch.cuda.synchronize()
+    return to_host(res)
+
+
+@pytest.mark.parametrize("case", KAT, ids=[c["name"] for c in KAT])
+def test_hand_derived_known_answers(case):
+    print("case", case["name"], flush=True)
+    got = run_gpu(case["rowPtr"], case["colIdx"], case["N"], case["W"])
+    want = dict(case)
+    want["tcbBitMap"] = np.array([int(x, 16) for x in case["tcbBitMap"]], dtype=np.uint64)
+    compare_preprocess(got, want)
+
+
+@pytest.mark.parametrize("W", [16, 8])
+@pytest.mark.parametrize("seed,N,deg,dup,unsorted,empty,hub", [
+    (0, 16, 3, False, False, 0.0, 0),
+    (1, 37, 4, False, False, 0.2, 0),
+    (2, 100, 9, True, True, 0.1, 7),
+    (3, 1030, 30, False, True, 0.0, 0),
+    (4, 64, 1, True, False, 0.6, 0),
+    (5, 2570, 12, True, True, 0.05, 9),
+    (6, 5000, 60, False, False, 0.0, 50),   # windows with > 512 TC blocks at W=8
+    (7, 20000, 2, False, False, 0.3, 0),
+])
+def test_random_graphs_bit_exact(oracle_mod, W, seed, N, deg, dup, unsorted, empty, hub):
+    print("case seed=%d N=%d W=%d" % (seed, N, W), flush=True)
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, dup=dup, unsorted=unsorted, empty_frac=empty, hub=hub)
+    got = run_gpu(rowPtr, colIdx, N, W)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N, 16, W)
+    compare_preprocess(got, want)
+
+
+def test_heavy_window_many_blocks(oracle_mod):
+    """One window whose rows name > 16*512 distinct columns: several LDS chunks in the fill."""
+    print("case heavy_window", flush=True)
+    rng = np.random.default_rng(0)
+    N = 40000
+    rows = []
+    for r in range(N):
+        if r < 16:
+            rows.append(np.sort(rng.choice(N, size=2500, replace=False)).astype(np.int32))
+        else:
+            rows.append(np.array([r], np.int32))
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum([len(x) for x in rows])
+    colIdx = np.concatenate(rows)
+    got = run_gpu(rowPtr, colIdx, N)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
+    assert want["blockPartition"][0] > 1024
+    compare_preprocess(got, want)
+
+
+def test_multi_pass_bitset_large_n(oracle_mod):
+    """N above the per-pass column range of the LDS bitset (393216) -> several passes."""
+    print("case large_n", flush=True)
+    from fused3s_amd import synth
+    N = 1_000_003
+    rp, ci = synth.rmat_graph(N, 3_000_000, 0.45, 0.22, 0.22, seed=1)
+    rowPtr, colIdx = rp.numpy(), ci.numpy()
+    got = run_gpu(rowPtr, colIdx, N)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
+    compare_preprocess(got, want)
+
+
+def test_empty_graph_and_tiny():
+    print("case empty", flush=True)
+    got = run_gpu(np.zeros(41, np.int32), np.zeros(0, np.int32), 40)
+    assert got["blockCount"] == 0 and list(got["rowWindowOffset"]) == [0, 0, 0, 0]
+    assert list(got["sortedRowWindows"]) == [0, 1, 2] and list(got["tcblockOffset"]) == [0]
+    got = run_gpu(np.array([0, 1], np.int32), np.array([0], np.int32), 1)
+    assert got["blockCount"] == 1 and got["sparseAToXidx"][0] == 0
+    assert int(got["tcbBitMap"][0]) == 1 << 63
+
+
+def test_out_of_range_column_is_an_error():
+    from fused3s_amd import capi
+    rp = torch.tensor([0, 1, 2], dtype=torch.int32).cuda()
+    ci = torch.tensor([0, 7], dtype=torch.int32).cuda()
+    with pytest.raises(RuntimeError, match="column index"):
+        capi.preprocess(rp, ci, 2)
+
+
+@pytest.mark.parametrize("name,scale", [("cfg1_gnm_2708", 1.0), ("cfg2_rmat_169k", 1.0),
+                                        ("cfg3_chunglu_233k", 0.02), ("cfg5_sbm_100k", 1.0)])
+def test_benchmark_shapes_bit_exact(oracle_mod, name, scale):
+    print("case", name, flush=True)
+    from fused3s_amd import synth
+    rp, ci = synth.make_graph(name, scale=scale)
+    N = rp.numel() - 1
+    got = run_gpu(rp.numpy(), ci.numpy(), N)
+    want = oracle_mod.preprocess(rp.numpy(), ci.numpy(), N)
+    compare_preprocess(got, want)
