@@ -58,8 +58,27 @@ __device__ __forceinline__ float row_sum4(float v) {
   return v;
 }
 
+// Everything one TC-block pair needs from memory, as it sits in registers.
+template <int D>
+struct PairData {
+  half8 kA[D / 32], kB[D / 32];            // K rows of the two blocks (A operand of S^T)
+  typename HalfVec<D / 16>::type vv[8];    // V pieces of this lane's 8 contraction slots
+  unsigned maskA, maskB;                   // bitmap byte holding this lane's 4 bits per block
+};
+// Metadata of a pair, one dword per lane from a single load: lanes 0..31 hold the 32 column ids
+// of blocks A and B, lanes 32..47 the 16 dwords of their bitmaps. Every lane later picks what it
+// needs with cross-lane reads, which do not go through the memory pipeline.
+struct PairIndex {
+  int meta;
+};
+
+// waves per SIMD the register allocator is held to: the two-stage pipeline needs ~170 VGPRs at
+// D = 64, and spilling costs more than the lost wave
+constexpr int waves_per_simd(int d) { return d <= 32 ? 4 : (d <= 64 ? 3 : 2); }
+
 template <int D, int NWAVES, bool SOFTMAX>
-__global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
+__global__ __launch_bounds__(NWAVES * 64)
+__attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
     int nRW, const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
@@ -107,40 +126,69 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
   const int maskByte = ((g >> 1) * 2 + (c >> 3)) * 8 + 7 - (c & 7);
   const int maskShift = 4 * (1 - (g & 1));
 
-  for (int p = wave; p < nPairs; p += NWAVES) {
-    const int tA = t0 + 2 * p;
+  // the second block of the window's last pair may not exist: it aliases the first one
+  // (loads stay in bounds) and its bits are cleared at use
+  auto load_index = [&](int p) {
+    const int64_t tA = t0 + 2 * p;
     const bool hasB = (tA + 1) < t1;
-    const int tB = hasB ? tA + 1 : tA;
-
-    // gathered K rows -> A operand
-    const int kRowA = sparseAToXidx[(int64_t)tA * 16 + c];
-    const int kRowB = sparseAToXidx[(int64_t)tB * 16 + c];
-    const half8* kpA = reinterpret_cast<const half8*>(K + (int64_t)kRowA * D) + g;
-    const half8* kpB = reinterpret_cast<const half8*>(K + (int64_t)kRowB * D) + g;
-    half8 kA[KS], kB[KS];
+    // lane -> dword index inside the pair's 32 ids / 16 bitmap dwords (second block folded onto
+    // the first when it does not exist)
+    const int idSlot = (lane & 31) & (hasB ? 31 : 15);
+    const int bmSlot = (lane & 15) & (hasB ? 15 : 7);
+    const int32_t* src = (lane < 32)
+                             ? sparseAToXidx + tA * 16 + idSlot
+                             : reinterpret_cast<const int32_t*>(bitmapBytes) + tA * 8 + bmSlot;
+    PairIndex ix;
+    ix.meta = *src;
+    return ix;
+  };
+  auto lane_read = [&](int v, int srcLane) { return __builtin_amdgcn_ds_bpermute(srcLane * 4, v); };
+  auto load_data = [&](const PairIndex& ix, int p) {
+    PairData<D> pd;
+    // 32-bit byte offsets from the uniform K / V bases (the launcher checks N*D*2 < 4 GiB): one
+    // address register per gathered row instead of a 64-bit pointer per load
+    const char* Kb = reinterpret_cast<const char*>(K);
+    const char* Vb = reinterpret_cast<const char*>(V);
+    // K is fetched with four adjacent lanes on one 64-byte piece of a row (lane -> slot lane/4,
+    // 16-byte chunk lane%4): 16 cache-line touches per load instead of 64. compute() moves the
+    // pieces to the MFMA layout (slot c, chunk g) with a cross-lane permute.
+    const uint32_t kRowA = (uint32_t)lane_read(ix.meta, lane >> 2);
+    const uint32_t kRowB = (uint32_t)lane_read(ix.meta, 16 + (lane >> 2));
+    const uint32_t koA = kRowA * (uint32_t)(D * 2) + (uint32_t)((lane & 3) * 16);
+    const uint32_t koB = kRowB * (uint32_t)(D * 2) + (uint32_t)((lane & 3) * 16);
 #pragma unroll
     for (int i = 0; i < KS; i++) {
-      kA[i] = kpA[4 * i];
-      kB[i] = kpB[4 * i];
+      pd.kA[i] = *reinterpret_cast<const half8*>(Kb + koA + 64 * i);
+      pd.kB[i] = *reinterpret_cast<const half8*>(Kb + koB + 64 * i);
     }
-    // V rows of this lane's 8 contraction slots
-    const int4 vIdxA = reinterpret_cast<const int4*>(sparseAToXidx + (int64_t)tA * 16)[g];
-    const int4 vIdxB = reinterpret_cast<const int4*>(sparseAToXidx + (int64_t)tB * 16)[g];
-    const int vr[8] = {vIdxA.x, vIdxA.y, vIdxA.z, vIdxA.w, vIdxB.x, vIdxB.y, vIdxB.z, vIdxB.w};
-    vrow_t vv[8];
 #pragma unroll
-    for (int k = 0; k < 8; k++)
-      vv[k] = reinterpret_cast<const vrow_t*>(V + (int64_t)vr[k] * D)[c];
-
-    unsigned bitsA = (bitmapBytes[(int64_t)tA * 32 + maskByte] >> maskShift) & 0xFu;
-    unsigned bitsB = (bitmapBytes[(int64_t)tB * 32 + maskByte] >> maskShift) & 0xFu;
-    if (!hasB) bitsB = 0;
-
+    for (int k = 0; k < 8; k++) {
+      const uint32_t vRow = (uint32_t)lane_read(ix.meta, (k < 4 ? 0 : 16) + 4 * g + (k & 3));
+      const uint32_t vo = vRow * (uint32_t)(D * 2) + (uint32_t)(c * T * 2);
+      pd.vv[k] = *reinterpret_cast<const vrow_t*>(Vb + vo);
+    }
+    pd.maskA = ((unsigned)lane_read(ix.meta, 32 + (maskByte >> 2)) >> (8 * (maskByte & 3))) & 0xFFu;
+    pd.maskB = ((unsigned)lane_read(ix.meta, 40 + (maskByte >> 2)) >> (8 * (maskByte & 3))) & 0xFFu;
+    return pd;
+  };
+  // lane (g, c) takes the 16 bytes that lane 4c + g loaded
+  const int permAddr = (4 * c + g) * 4;
+  auto to_mfma_layout = [&](half8 v) {
+    typedef int int4v __attribute__((ext_vector_type(4)));
+    int4v x = __builtin_bit_cast(int4v, v);
+#pragma unroll
+    for (int k = 0; k < 4; k++) x[k] = __builtin_amdgcn_ds_bpermute(permAddr, x[k]);
+    return __builtin_bit_cast(half8, x);
+  };
+  auto compute = [&](const PairData<D>& pd, int p) {
+    const bool hasB = (t0 + 2 * p + 1) < t1;
+    const unsigned bitsA = (pd.maskA >> maskShift) & 0xFu;
+    const unsigned bitsB = hasB ? ((pd.maskB >> maskShift) & 0xFu) : 0u;
     float4v sA = {0.f, 0.f, 0.f, 0.f}, sB = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < KS; i++) {
-      sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kA[i], qf[i], sA, 0, 0, 0);
-      sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kB[i], qf[i], sB, 0, 0, 0);
+      sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_mfma_layout(pd.kA[i]), qf[i], sA, 0, 0, 0);
+      sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_mfma_layout(pd.kB[i]), qf[i], sB, 0, 0, 0);
     }
     float s[8];
 #pragma unroll
@@ -148,7 +196,6 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
       s[i] = ((bitsA >> (3 - i)) & 1u) ? sA[i] : 0.0f;
       s[4 + i] = ((bitsB >> (3 - i)) & 1u) ? sB[i] : 0.0f;
     }
-
     half8 pf;
     if constexpr (SOFTMAX) {
       float mx = m;
@@ -174,13 +221,33 @@ __global__ __launch_bounds__(NWAVES * 64) void f3s_fwd_kernel(
 #pragma unroll
       for (int i = 0; i < 8; i++) pf[i] = (_Float16)s[i];
     }
-
 #pragma unroll
     for (int j = 0; j < T; j++) {
       half8 va;
 #pragma unroll
-      for (int k = 0; k < 8; k++) va[k] = vv[k][j];
+      for (int k = 0; k < 8; k++) va[k] = pd.vv[k][j];
       o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pf, o[j], 0, 0, 0);
+    }
+  };
+
+  // Two-stage software pipeline per wave: while pair p is computed, the K/V rows of the wave's
+  // next pair and the indices of the one after are already in flight.
+  int p = wave;
+  if (p < nPairs) {
+    PairIndex ixA = load_index(p), ixB;
+    PairData<D> pdA = load_data(ixA, p), pdB;
+    if (p + NWAVES < nPairs) ixB = load_index(p + NWAVES);
+    while (true) {
+      if (p + NWAVES < nPairs) pdB = load_data(ixB, p + NWAVES);
+      if (p + 2 * NWAVES < nPairs) ixA = load_index(p + 2 * NWAVES);
+      compute(pdA, p);
+      p += NWAVES;
+      if (p >= nPairs) break;
+      if (p + NWAVES < nPairs) pdA = load_data(ixA, p + NWAVES);
+      if (p + 2 * NWAVES < nPairs) ixB = load_index(p + 2 * NWAVES);
+      compute(pdB, p);
+      p += NWAVES;
+      if (p >= nPairs) break;
     }
   }
 
@@ -262,6 +329,8 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   if (dtype != 0) return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16)", dtype);
   if (cuTimer) return fail(-3, "f3s_attention_fwd: per-CU timing not supported yet");
   if (scalingFactor == 0.0f) return fail(-2, "f3s_attention_fwd: scalingFactor must be non-zero");
+  if ((int64_t)N * d * 2 >= (int64_t)1 << 32)
+    return fail(-2, "f3s_attention_fwd: K and V must each be smaller than 4 GiB (N*d*2 bytes)");
   // the reference divides unmasked scores by scalingFactor (src/F3S_kernel.cu:1666-1667);
   // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;

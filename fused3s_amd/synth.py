@@ -64,9 +64,20 @@ def _rmat_edges(n, scale, a, b, c, g, device):
     return src, dst
 
 
+def _relabel(keys, N, g, device):
+    """Apply one random vertex permutation to both endpoints of the packed (src*N+dst) keys, so
+    that hubs are spread over the row windows as in a real dataset instead of sitting in the
+    first rows (R-MAT and Chung-Lu both emit hubs at low ids)."""
+    perm = torch.randperm(N, generator=g, device=device)
+    src = torch.div(keys, N, rounding_mode="floor")
+    dst = keys - src * N
+    return perm[src], perm[dst]
+
+
 def rmat_graph(N, target_edges, a, b, c, seed=0, device="cpu", max_rounds=12):
     """R-MAT over 2^ceil(log2 N) ids, ids >= N rejected, drawn until the symmetrised, deduped
-    edge set (self-loops included) reaches ~target_edges. Configurations 2 and 4."""
+    edge set (self-loops included) reaches ~target_edges; vertices are then relabelled by a
+    random permutation. Configurations 2 and 4."""
     g = _gen(seed, device)
     scale = max(1, math.ceil(math.log2(N)))
     keys = torch.empty(0, dtype=torch.int64, device=device)
@@ -80,8 +91,7 @@ def rmat_graph(N, target_edges, a, b, c, seed=0, device="cpu", max_rounds=12):
         need = target_edges - N - int(keys.numel())
         if need <= 0.01 * target_edges:
             break
-    src = torch.div(keys, N, rounding_mode="floor")
-    dst = keys - src * N
+    src, dst = _relabel(keys, N, g, device)
     return edges_to_csr(src, dst, N, symmetrize=False)
 
 
@@ -89,7 +99,8 @@ def chung_lu_graph(N, target_edges, gamma=2.1, max_degree=22000, seed=0, device=
                    max_rounds=12):
     """Chung-Lu: endpoints drawn independently with probability proportional to the weights
     w_i = (i + i0)^(-1/(gamma-1)), i0 chosen so that w_max / mean(w) = max_degree / mean degree;
-    pairs are symmetrised and deduped until ~target_edges directed edges (self-loops included).
+    pairs are symmetrised and deduped until ~target_edges directed edges (self-loops included),
+    then vertices are relabelled by a random permutation.
     Configuration 3."""
     g = _gen(seed, device)
     alpha = 1.0 / (gamma - 1.0)
@@ -123,8 +134,7 @@ def chung_lu_graph(N, target_edges, gamma=2.1, max_degree=22000, seed=0, device=
         need = target_edges - N - int(keys.numel())
         if need <= 0.01 * target_edges:
             break
-    src = torch.div(keys, N, rounding_mode="floor")
-    dst = keys - src * N
+    src, dst = _relabel(keys, N, g, device)
     return edges_to_csr(src, dst, N, symmetrize=False)
 
 

@@ -50,7 +50,7 @@ def lib():
                                                ctypes.c_float, ci, ci, ci, ci, f32p]
         L.f3s_oracle_attention_textbook.restype = ci
         L.f3s_oracle_attention_textbook.argtypes = [i32p, i32p, ci, ci, ci, u16p, u16p, u16p,
-                                                    ctypes.c_float, ci, ci, f32p]
+                                                    ctypes.c_float, ci, ci, ci, f32p]
         L.f3s_oracle_half_to_float.restype = ctypes.c_float
         L.f3s_oracle_half_to_float.argtypes = [ctypes.c_uint16]
         L.f3s_oracle_round_to_half.restype = ctypes.c_float
@@ -132,8 +132,10 @@ def attention_ref(rwo, atox, bitmap, N, Q, K, V, scalingFactor=1.0, nWarpPerBloc
     return out
 
 
-def attention_textbook(rowPtr, colIdx, N, Q, K, V, scalingFactor=1.0, dtype=0, rows=None):
-    """Textbook masked softmax attention from CSR, fp64 accumulate."""
+def attention_textbook(rowPtr, colIdx, N, Q, K, V, scalingFactor=1.0, dtype=0, rows=None,
+                       row_step=1):
+    """Textbook masked softmax attention from CSR, fp64 accumulate. rows=(begin, end) and
+    row_step restrict the computation to rows begin, begin+row_step, ... < end."""
     L = lib()
     Qb, Kb, Vb = _bits(Q), _bits(K), _bits(V)
     d = Qb.shape[1]
@@ -144,7 +146,8 @@ def attention_textbook(rowPtr, colIdx, N, Q, K, V, scalingFactor=1.0, dtype=0, r
     rc = L.f3s_oracle_attention_textbook(_p(rowPtr, ctypes.c_int32), _p(colIdx, ctypes.c_int32),
                                          N, d, dtype, _p(Qb, ctypes.c_uint16),
                                          _p(Kb, ctypes.c_uint16), _p(Vb, ctypes.c_uint16),
-                                         float(scalingFactor), rb, re, _p(out, ctypes.c_float))
+                                         float(scalingFactor), rb, re, int(row_step),
+                                         _p(out, ctypes.c_float))
     assert rc == 0, rc
     return out
 

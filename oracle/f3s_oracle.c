@@ -420,12 +420,14 @@ int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *spar
  * N(i) = DISTINCT columns of CSR row i, empty row => 0.
  *   row_wise_softmax_mask followed by S @ V   scripts/tests/test_f3s_accuracy.py:81-94,148-164
  *   edge-wise SDDMM / segment softmax / SpMM  scripts/baseline_comp/baseline_comp_kernel_only.py:667-686
- * Rows [rowBegin,rowEnd) only, so a bounded sample of a large graph can be checked or timed.
+ * Rows rowBegin, rowBegin+rowStep, ... < rowEnd only, so a bounded, evenly spaced sample of a
+ * large graph can be checked or timed.
  */
 int f3s_oracle_attention_textbook(const int32_t *rowPtr, const int32_t *colIdx, int N, int d,
                                   int dtype, const uint16_t *Q, const uint16_t *K,
                                   const uint16_t *V, float scalingFactor, int rowBegin,
-                                  int rowEnd, float *out) {
+                                  int rowEnd, int rowStep, float *out) {
+  if (rowStep < 1) rowStep = 1;
   if (rowBegin < 0) rowBegin = 0;
   if (rowEnd > N || rowEnd < 0) rowEnd = N;
   float *Qf = to_float(Q, (int64_t)N * d, dtype);
@@ -440,7 +442,7 @@ int f3s_oracle_attention_textbook(const int32_t *rowPtr, const int32_t *colIdx, 
     double *sc = (double *)malloc(sizeof(double) * (size_t)cap);
     double *acc = (double *)malloc(sizeof(double) * (size_t)d);
 #pragma omp for schedule(dynamic, 16)
-    for (int r = rowBegin; r < rowEnd; r++) {
+    for (int r = rowBegin; r < rowEnd; r += rowStep) {
       int64_t s = rowPtr[r], e = rowPtr[r + 1];
       int64_t n = e - s;
       float *o = out + (int64_t)r * d;
