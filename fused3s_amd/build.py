@@ -56,7 +56,7 @@ def build_extension():
         cmd += ["-isystem", i]
     cmd += [os.path.join(CSRC, "f3s_torch.cpp"), "-o", EXT_PATH,
             "-L" + HERE, "-lf3s_amd", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu",
-            "-ltorch_hip", "-ltorch", "-ltorch_python",
+            "-ltorch_hip", "-ltorch", "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
             "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib]
     _run(cmd)
     return EXT_PATH

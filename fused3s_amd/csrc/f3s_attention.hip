@@ -76,14 +76,30 @@ struct PairIndex {
 // D = 64, and spilling costs more than the lost wave
 constexpr int waves_per_simd(int d) { return d <= 32 ? 4 : (d <= 64 ? 3 : 2); }
 
-template <int D, int NWAVES, bool SOFTMAX>
+// Constant-rate (100 MHz) timestamp shared by all CUs, and an id of the CU this wave runs on:
+// XCC id in bits 8.., {SE, SH, CU} of HW_ID in bits 0..7. Used only by the timed variant, which
+// replaces the reference's %globaltimer / %smid reads (src/F3S_kernel.cu:30-40).
+__device__ __forceinline__ unsigned long long realtime_ticks() {
+  return __builtin_amdgcn_s_memrealtime();
+}
+__device__ __forceinline__ unsigned cu_key() {
+  unsigned hw, xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  return ((xcc & 0xFu) << 8) | ((hw >> 8) & 0xFFu);
+}
+
+template <int D, int NWAVES, bool SOFTMAX, bool CLOCKED>
 __global__ __launch_bounds__(NWAVES * 64)
 __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
     int nRW, const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
-    const _Float16* __restrict__ V, float scaleLog2, float* __restrict__ out) {
+    const _Float16* __restrict__ V, float scaleLog2, float* __restrict__ out,
+    unsigned long long* __restrict__ cuTimer) {
   constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
+  unsigned long long tBegin = 0;
+  if constexpr (CLOCKED) tBegin = realtime_ticks();
   constexpr int KS = D / 32;  // MFMA k-steps of the score product
   constexpr int OSTRIDE = D + 4;
   typedef typename HalfVec<T>::type vrow_t;
@@ -302,19 +318,35 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     }
     *reinterpret_cast<float4*>(out + row * D + cv * 4) = acc;
   }
+  if constexpr (CLOCKED) {
+    // {first tick, last tick, CU} of this workgroup, as the reference's timed kernels record
+    // {begin, end, smid} per block (src/F3S_kernel.cu:1363-1367)
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      cuTimer[3 * (size_t)blockIdx.x + 0] = tBegin;
+      cuTimer[3 * (size_t)blockIdx.x + 1] = realtime_ticks();
+      cuTimer[3 * (size_t)blockIdx.x + 2] = cu_key();
+    }
+  }
 }
 
 template <int D, bool SOFTMAX>
 int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, const uint64_t* bitmap,
              int N, const void* Q, const void* K, const void* V, float scaleLog2, float* out,
-             hipStream_t stream) {
+             unsigned long long* cuTimer, hipStream_t stream) {
   constexpr int NWAVES = 4;
   const int nRW = (N + kWinRows - 1) / kWinRows;
   if (nRW == 0) return 0;
-  hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX>), dim3(nRW), dim3(NWAVES * 64), 0, stream,
-                     rwo, order, atox, reinterpret_cast<const uint8_t*>(bitmap), N, nRW,
-                     static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
-                     static_cast<const _Float16*>(V), scaleLog2, out);
+  const auto* bm = reinterpret_cast<const uint8_t*>(bitmap);
+  const auto* q = static_cast<const _Float16*>(Q);
+  const auto* k = static_cast<const _Float16*>(K);
+  const auto* v = static_cast<const _Float16*>(V);
+  if (cuTimer)
+    hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX, true>), dim3(nRW), dim3(NWAVES * 64), 0,
+                       stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer);
+  else
+    hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX, false>), dim3(nRW), dim3(NWAVES * 64),
+                       0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -327,7 +359,6 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                      int applySoftmax, float* out, unsigned long long* cuTimer,
                      hipStream_t stream) {
   if (dtype != 0) return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16)", dtype);
-  if (cuTimer) return fail(-3, "f3s_attention_fwd: per-CU timing not supported yet");
   if (scalingFactor == 0.0f) return fail(-2, "f3s_attention_fwd: scalingFactor must be non-zero");
   if ((int64_t)N * d * 2 >= (int64_t)1 << 32)
     return fail(-2, "f3s_attention_fwd: K and V must each be smaller than 4 GiB (N*d*2 bytes)");
@@ -337,9 +368,11 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
 #define F3S_DISPATCH(DD)                                                                       \
   case DD:                                                                                     \
     return applySoftmax ? launch_d<DD, true>(rowWindowOffset, windowOrder, sparseAToXidx,      \
-                                             bitmap, N, Q, K, V, scaleLog2, out, stream)       \
+                                             bitmap, N, Q, K, V, scaleLog2, out, cuTimer,      \
+                                             stream)                                           \
                         : launch_d<DD, false>(rowWindowOffset, windowOrder, sparseAToXidx,     \
-                                              bitmap, N, Q, K, V, scaleLog2, out, stream);
+                                              bitmap, N, Q, K, V, scaleLog2, out, cuTimer,     \
+                                              stream);
   switch (d) {
     F3S_DISPATCH(32)
     F3S_DISPATCH(64)

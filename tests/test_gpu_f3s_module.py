@@ -1,0 +1,127 @@
+"""The `F3S` operator module used the way the reference's callers use it
+(scripts/tests/test_f3s_accuracy.py:96-236, scripts/baseline_comp/baseline_comp_kernel_only.py:
+412-497): preprocess_gpu on CSR, then each fused entry point, checked against the oracles."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from ref_checks import compare_preprocess, dense_attention
+
+pytestmark = pytest.mark.gpu
+MAX_ABS = 2e-2
+MEAN_REL = 1e-3
+
+
+def reference_style_inputs(N=1000, d=128, density=0.1, seed=0):
+    rng = np.random.default_rng(seed)
+    A = rng.random((N, N)) < density
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(A.sum(axis=1))
+    colIdx = np.nonzero(A)[1].astype(np.int32)
+    Q, K, V = [rng.random((N, d)).astype(np.float16) for _ in range(3)]
+    return rowPtr, colIdx, Q, K, V
+
+
+def preprocess_like_the_reference(F3S, rowPtr, colIdx, N, W=16):
+    dev = "cuda"
+    nRW = (N + 15) // 16
+    blockPartition = torch.zeros(nRW, dtype=torch.int32, device=dev)
+    edgeToColumn = torch.zeros(len(colIdx), dtype=torch.int32, device=dev)
+    edgeToRow = torch.zeros(len(colIdx), dtype=torch.int32, device=dev)
+    res = F3S.preprocess_gpu(torch.as_tensor(colIdx).to(dev), torch.as_tensor(rowPtr).to(dev), N,
+                             16, W, blockPartition, edgeToColumn, edgeToRow)
+    return res, blockPartition, edgeToColumn, edgeToRow
+
+
+def test_reference_call_sequence_all_variants(oracle_mod, tmp_path, monkeypatch):
+    print("case module_all_variants", flush=True)
+    from fused3s_amd import F3S
+    monkeypatch.chdir(tmp_path)
+    N, d = 1000, 128
+    rowPtr, colIdx, Q, K, V = reference_style_inputs(N, d)
+    res, blockPartition, edgeToColumn, edgeToRow = preprocess_like_the_reference(
+        F3S, rowPtr, colIdx, N)
+    rwo, order, rowid, tile, toff, atox, bm, count = res
+    assert isinstance(count, int) and count == atox.numel() // 16
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
+    got = dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
+               tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox, blockCount=count,
+               tcbBitMap=bm.cpu().view(torch.int64).numpy().view(np.uint64),
+               blockPartition=blockPartition, edgeToColumn=edgeToColumn, edgeToRow=edgeToRow)
+    got = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in got.items()}
+    compare_preprocess(got, want)
+
+    Qd, Kd, Vd = (torch.as_tensor(x).cuda() for x in (Q, K, V))
+    true = dense_attention(rowPtr, colIdx, N, Q, K, V, 1.0)
+    ref = oracle_mod.attention_ref(want["rowWindowOffset"], want["sparseAToXidx"],
+                                   want["tcbBitMap"], N, Q, K, V, 1.0)
+    outs = {
+        "f3s_1tb1rw": F3S.f3s_1tb1rw(rwo, atox, bm, N, Qd, Kd, Vd, 8, True, False),
+        "f3s_1tb1rw_scheduled": F3S.f3s_1tb1rw_scheduled(rwo, order, atox, bm, N, Qd, Kd, Vd, 8,
+                                                         False),
+        "f3s_1tb1rw_scheduled_permuteV": F3S.f3s_1tb1rw_scheduled_permuteV(rwo, order, atox, bm,
+                                                                           N, Qd, Kd, Vd, 8),
+        "scaleQK_1.0": F3S.f3s_1tb1rw_scheduled_permuteV_scaleQK(rwo, order, atox, bm, N, Qd, Kd,
+                                                                 Vd, 1.0, 8),
+    }
+    for name, r in outs.items():
+        time_ms, out, sddmm = r
+        assert time_ms.dim() == 0 and time_ms.device.type == "cpu" and float(time_ms) > 0
+        assert out.shape == (N, d) and out.dtype == torch.float32 and out.is_cuda
+        assert sddmm.numel() == 0
+        o = out.cpu().numpy()
+        # the reference's own figure of merit: relative Frobenius error against dense fp32/64
+        assert np.linalg.norm(o - true) / np.linalg.norm(true) < 2e-3, name
+        assert np.abs(o - ref).max() < MAX_ABS, name
+
+    # scaled variant: scores divided by scalingFactor
+    scale = float(np.sqrt(d))
+    r = F3S.f3s_1tb1rw_scheduled_permuteV_scaleQK(rwo, order, atox, bm, N, Qd, Kd, Vd, scale, 8)
+    want_s = oracle_mod.attention_ref(want["rowWindowOffset"], want["sparseAToXidx"],
+                                      want["tcbBitMap"], N, Q, K, V, scale)
+    o = r[1].cpu().numpy()
+    assert np.abs(o - want_s).max() < MAX_ABS
+    assert np.abs(o - want_s).mean() / np.abs(want_s).mean() < MEAN_REL
+
+    # SDDMM -> SpMM without softmax
+    r = F3S.f3s_1tb1rw(rwo, atox, bm, N, Qd, Kd, Vd, 8, False, False)
+    want_n = oracle_mod.attention_ref(want["rowWindowOffset"], want["sparseAToXidx"],
+                                      want["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
+    o = r[1].cpu().numpy()
+    assert np.abs(o - want_n).max() < 2e-2 * np.abs(want_n).max()
+
+    # per-CU active time files of the timed variants (reference: one "begin end" line per SM)
+    F3S.f3s_1tb1rw(rwo, atox, bm, N, Qd, Kd, Vd, 8, True, True)
+    F3S.f3s_1tb1rw_scheduled(rwo, order, atox, bm, N, Qd, Kd, Vd, 8, True)
+    for fn in ("SM_time_f3s1tb1rw.csv", "SM_time_f3s1tb1rw_scheduled.csv"):
+        lines = open(os.path.join(tmp_path, fn)).read().split("\n")
+        rows = [l.split() for l in lines if l.strip()]
+        assert 1 <= len(rows) <= 256
+        for b, e in rows:
+            assert float(e) >= float(b) > 0
+
+
+def test_module_argument_checks_on_device():
+    print("case module_arg_checks", flush=True)
+    from fused3s_amd import F3S
+    N, d = 64, 64
+    rwo = torch.zeros(5, dtype=torch.int32, device="cuda")
+    atox = torch.zeros(16, dtype=torch.int32, device="cuda")
+    bm = torch.zeros(4, dtype=torch.uint64, device="cuda")
+    Q = torch.zeros(N, d, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="contiguous"):
+        F3S.f3s_1tb1rw(rwo, atox, bm, N, Q.t().contiguous().t(), Q, Q, 8, True, False)
+    with pytest.raises(RuntimeError, match="float16"):
+        F3S.f3s_1tb1rw(rwo, atox, bm, N, Q.float(), Q.float(), Q.float(), 8, True, False)
+    with pytest.raises(RuntimeError, match="nWarpPerBlock"):
+        F3S.f3s_1tb1rw(rwo, atox, bm, N, Q, Q, Q, 3, True, False)
+    Qbad = torch.zeros(N, 48, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="head dim"):
+        F3S.f3s_1tb1rw(rwo, atox, bm, N, Qbad, Qbad, Qbad, 8, True, False)
+    with pytest.raises(RuntimeError, match="not implemented"):
+        F3S.f3s_1tb1tcb(rwo, atox, bm, N, Q, Q, Q, True, False)
+    # all-empty graph: every output row is zero
+    out = F3S.f3s_1tb1rw(rwo, atox, bm, N, Q, Q, Q, 8, True, False)[1]
+    assert float(out.abs().max()) == 0.0
