@@ -10,7 +10,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libf3s_amd.so")
+LIB_PATH = os.environ.get("F3S_AMD_LIB", os.path.join(_HERE, "libf3s_amd.so"))
 _lib = None
 
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
