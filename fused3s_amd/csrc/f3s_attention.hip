@@ -72,9 +72,11 @@ struct PairIndex {
   int meta;
 };
 
-// waves per SIMD the register allocator is held to: the two-stage pipeline needs ~170 VGPRs at
-// D = 64, and spilling costs more than the lost wave
-constexpr int waves_per_simd(int d) { return d <= 32 ? 4 : (d <= 64 ? 3 : 2); }
+// Waves per SIMD the kernel is held to. Two, not more: with three or four waves per SIMD the
+// extra windows in flight per XCD spread the K/V rows being gathered over more of the column
+// range than the 4 MiB L2 covers, and the kernel gets slower (measured 2.0 ms at two waves,
+// 2.6 ms at three on the 233k-node benchmark graph).
+constexpr int waves_per_simd(int d) { return d <= 32 ? 4 : 2; }
 
 // Constant-rate (100 MHz) timestamp shared by all CUs, and an id of the CU this wave runs on:
 // XCC id in bits 8.., {SE, SH, CU} of HW_ID in bits 0..7. Used only by the timed variant, which
@@ -159,7 +161,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     return ix;
   };
   auto lane_read = [&](int v, int srcLane) { return __builtin_amdgcn_ds_bpermute(srcLane * 4, v); };
-  auto load_data = [&](const PairIndex& ix, int p) {
+  auto load_data = [&](const PairIndex& ix) {
     PairData<D> pd;
     // 32-bit byte offsets from the uniform K / V bases (the launcher checks N*D*2 < 4 GiB): one
     // address register per gathered row instead of a 64-bit pointer per load
@@ -246,25 +248,35 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     }
   };
 
-  // Two-stage software pipeline per wave: while pair p is computed, the K/V rows of the wave's
-  // next pair and the indices of the one after are already in flight.
-  int p = wave;
-  if (p < nPairs) {
-    PairIndex ixA = load_index(p), ixB;
-    PairData<D> pdA = load_data(ixA, p), pdB;
-    if (p + NWAVES < nPairs) ixB = load_index(p + NWAVES);
+  // Software pipeline per wave over its pairs p = wave, wave + NWAVES, ...: in the step of pair p
+  // the metadata of pair p+4 is requested, the K/V loads of pair p+2 are issued (their metadata
+  // was requested four steps earlier, so waiting for it never waits for younger K/V loads and
+  // the cold HBM miss it usually is stays off the critical path), and pair p is computed.
+  // Three data buffers and three metadata registers rotate; the loop is unrolled three times so
+  // that every buffer has a fixed role in every copy of the body.
+  if (wave < nPairs) {
+    // loads past the wave's last pair are redirected to that pair (same lines again, no branch)
+    const int pLast = wave + ((nPairs - 1 - wave) / NWAVES) * NWAVES;
+    auto clamp_pair = [&](int q) { return q < pLast ? q : pLast; };
+    int p = wave;
+    PairIndex m0 = load_index(p);
+    PairIndex m1 = load_index(clamp_pair(p + NWAVES));
+    PairIndex m2 = load_index(clamp_pair(p + 2 * NWAVES));
+    PairData<D> pd0 = load_data(m0), pd1, pd2;
+    m0 = load_index(clamp_pair(p + 3 * NWAVES));
+    pd1 = load_data(m1);
+#define F3S_STEP(CUR, FILL, MUSE, MFILL)              \
+  MFILL = load_index(clamp_pair(p + 4 * NWAVES));      \
+  FILL = load_data(MUSE);                              \
+  compute(CUR, p);                                     \
+  p += NWAVES;                                         \
+  if (p > pLast) break;
     while (true) {
-      if (p + NWAVES < nPairs) pdB = load_data(ixB, p + NWAVES);
-      if (p + 2 * NWAVES < nPairs) ixA = load_index(p + 2 * NWAVES);
-      compute(pdA, p);
-      p += NWAVES;
-      if (p >= nPairs) break;
-      if (p + NWAVES < nPairs) pdA = load_data(ixA, p + NWAVES);
-      if (p + 2 * NWAVES < nPairs) ixB = load_index(p + 2 * NWAVES);
-      compute(pdB, p);
-      p += NWAVES;
-      if (p >= nPairs) break;
+      F3S_STEP(pd0, pd2, m2, m1)
+      F3S_STEP(pd1, pd0, m0, m2)
+      F3S_STEP(pd2, pd1, m1, m0)
     }
+#undef F3S_STEP
   }
 
   // ---- merge the waves' partial (m, l, O) and write the window's rows
