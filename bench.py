@@ -79,6 +79,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
     ap.add_argument("--cpu-budget", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (row windows would shard across GPUs with K/V "
@@ -123,6 +126,14 @@ def main():
     cnt = (pre["rowWindowOffset"][1:] - pre["rowWindowOffset"][:-1])
     log("preprocess: nTCB=%d nRW=%d max TCB/window=%d mean=%.1f  %.2f ms (%.2f G edges/s)"
         % (nTCB, nRW, int(cnt.max()), float(cnt.float().mean()), pre_ms, E / pre_ms / 1e6))
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     order = None if args.natural_order else pre["sortedRowWindows"]
     out = torch.empty((N, d), dtype=torch.float32, device=dev)
