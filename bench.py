@@ -69,6 +69,17 @@ def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
                       "(%d rows, %d edges), %.1f s wall" % (step, rows_done, edges, spent)}
 
 
+def measured_traffic(args):
+    """HBM-side bytes per launch of the attention kernel from rocprofv3 (FETCH_SIZE x 2.000 +
+    WRITE_SIZE x 1.000, factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md).
+    Counters cannot be read from inside this process, so the figure is the recorded one and is
+    only given for the workload it was measured on."""
+    if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
+        return {"bytes_per_launch": 14_644_661 * 1024, "source": "rocprofv3 --pmc FETCH_SIZE / "
+                "WRITE_SIZE, see profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md"}
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -183,7 +194,8 @@ def main():
         "gather_gbps": b_gather / t_med / 1e9,
         "preprocess_ms": pre_ms, "preprocess_gedges_per_s": E / pre_ms / 1e6,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS,
+                     "traffic": measured_traffic(args)},
     }
     log("kernel: median %.3f ms  mean %.3f ms  effective %.1f TFLOP/s  MFMA %.1f TFLOP/s (%.1f%%)"
         % (t_med * 1e3, t_avg * 1e3, f_eff / t_med / 1e12, achieved,
