@@ -75,8 +75,7 @@ def measured_traffic(args):
     Counters cannot be read from inside this process, so the figure is the recorded one and is
     only given for the workload it was measured on."""
     if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
-        return {"bytes_per_launch": 14_644_661 * 1024, "source": "rocprofv3 --pmc FETCH_SIZE / "
-                "WRITE_SIZE, see profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md"}
+        return 14_644_661 * 1024
     return None
 
 

@@ -4,7 +4,11 @@
 // a global thrust::sort of (window, column) pairs followed by two kernels that walk each
 // window with a single thread. Here a window never leaves its workgroup:
 //
-//   window_rank_kernel   one workgroup per window. Column ids are OR-ed into an LDS bitset
+//   window_rank_small_kernel  windows of <= 1024 edges, one WAVE per window: bitonic sort of the
+//                        column ids in LDS, ballot / popcount compaction of the distinct ones,
+//                        rank by binary search. No workgroup barrier.
+//   window_rank_kernel   larger windows, one workgroup per window. Column ids are OR-ed into an
+//                        LDS bitset
 //                        (a column range per pass when N exceeds the LDS range), a wave64
 //                        popcount prefix scan turns the bitset into ranks, and every edge
 //                        reads its compacted column index back: the sorted unique column list
@@ -26,6 +30,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kRangeMax = 393216;  // columns per bitset pass: 48 KiB of bits + 12 KiB of prefixes
+constexpr int kSortMax = 1024;     // windows up to this many edges are ranked by a per-wave LDS sort
 constexpr int kFillChunk = 512;    // TC blocks held in LDS at once by window_fill_kernel
 
 // workspace header (bytes 0..255): int64 nTCB, int32 error flag
@@ -55,10 +60,139 @@ __device__ __forceinline__ int row_of_edge(const int* sRow, int e) {
 }
 
 // ------------------------------------------------------------------ phase 1
+// compiler-level ordering point between LDS phases of ONE wave (its LDS operations execute in
+// program order, so no hardware barrier is needed)
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_wave_barrier();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
+// Windows of at most kSortMax edges: one WAVE per window, no workgroup barrier. The wave sorts
+// the window's column ids in its LDS slice (bitonic network, 32 compare-exchanges per step and
+// lane row), compacts the distinct ones with ballot + popcount prefixes, and ranks every edge by
+// binary search in the distinct list.
+template <int W>
+__global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int nRW,
+    int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr) {
+  constexpr int WAVES = kBlock / 64;
+  __shared__ uint32_t sKeys[WAVES][kSortMax];
+  __shared__ uint32_t sUniq[WAVES][kSortMax];
+  __shared__ int sRowW[WAVES][17];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int w = blockIdx.x * WAVES + wave;
+  if (w >= nRW) return;
+  const int r0 = w * 16;
+  int* sRow = sRowW[wave];
+  if (lane < 17) sRow[lane] = rowPtr[min(r0 + lane, N)];
+  wave_lds_sync();
+  const int eS = sRow[0], eE = sRow[16];
+  const int n = eE - eS;
+  if (n == 0) {
+    if (lane == 0) blockPartition[w] = 0;
+    return;
+  }
+  if (n > kSortMax) return;  // ranked by window_rank_kernel
+  uint32_t* keys = sKeys[wave];
+  uint32_t* uniq = sUniq[wave];
+  int P = 64;
+  while (P < n) P <<= 1;
+  bool bad = false;
+  for (int i = lane; i < P; i += 64) {
+    uint32_t k = 0xFFFFFFFFu;  // padding sorts last
+    if (i < n) {
+      k = (uint32_t)colIdx[eS + i];
+      if (k >= (uint32_t)N) {
+        bad = true;
+        k = 0xFFFFFFFEu;
+      }
+    }
+    keys[i] = k;
+  }
+  if (bad) atomicOr(&hdr->error, 1);
+  wave_lds_sync();
+  for (int k = 2; k <= P; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      // all of the lane's compare-exchanges of this step: reads first, then writes, so the
+      // LDS latencies overlap (at most kSortMax / 128 pairs per lane)
+      constexpr int MAXP = kSortMax / 128;
+      uint32_t va[MAXP], vb[MAXP];
+      const int nPairsLane = P >> 7;  // P/2 pairs over 64 lanes (P >= 128), 0 when P == 64
+      if (nPairsLane == 0) {
+        if (lane < 32) {
+          const int lo = ((lane & ~(j - 1)) << 1) | (lane & (j - 1));
+          const int hi = lo | j;
+          const uint32_t x = keys[lo], y = keys[hi];
+          const bool up = (lo & k) == 0;
+          if ((x > y) == up) {
+            keys[lo] = y;
+            keys[hi] = x;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < MAXP; q++) {
+          if (q < nPairsLane) {
+            const int i = lane + 64 * q;
+            const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+            va[q] = keys[lo];
+            vb[q] = keys[lo | j];
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < MAXP; q++) {
+          if (q < nPairsLane) {
+            const int i = lane + 64 * q;
+            const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+            const bool up = (lo & k) == 0;
+            const bool swap = (va[q] > vb[q]) == up;
+            keys[lo] = swap ? vb[q] : va[q];
+            keys[lo | j] = swap ? va[q] : vb[q];
+          }
+        }
+      }
+      wave_lds_sync();
+    }
+  }
+  int nUniq = 0;
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  for (int base = 0; base < P; base += 64) {
+    const int i = base + lane;
+    const uint32_t k = keys[i];
+    const bool first = k < 0xFFFFFFFEu && (i == 0 || keys[i - 1] != k);
+    const unsigned long long bal = __ballot(first);
+    if (first) uniq[nUniq + __popcll(bal & ltMask)] = k;
+    nUniq += __popcll(bal);
+  }
+  wave_lds_sync();
+  for (int e = eS + lane; e < eE; e += 64) {
+    const uint32_t col = (uint32_t)colIdx[e];
+    int lo = 0, hi = nUniq - 1, found = 0;
+    while (lo <= hi) {
+      const int mid = (lo + hi) >> 1;
+      const uint32_t v = uniq[mid];
+      if (v == col) {
+        found = mid;
+        break;
+      }
+      if (v < col)
+        lo = mid + 1;
+      else
+        hi = mid - 1;
+    }
+    edgeToColumn[e] = found;
+    edgeToRow[e] = r0 + row_of_edge(sRow, e);
+  }
+  if (lane == 0) blockPartition[w] = (nUniq + W - 1) / W;
+}
+
 template <int W>
 __global__ __launch_bounds__(kBlock) void window_rank_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
-    int nPasses, int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
+    int nPasses, int sortMax, int32_t* __restrict__ blockPartition,
+    int32_t* __restrict__ edgeToColumn,
     int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr) {
   extern __shared__ __align__(16) uint32_t smem[];
   uint32_t* bits = smem;                 // range/32 words
@@ -78,6 +212,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
     if (tid == 0) blockPartition[w] = 0;
     return;
   }
+  if (eE - eS <= sortMax) return;  // ranked by window_rank_small_kernel
   const int nGroups = range >> 7;
   unsigned uniqueBefore = 0;
   for (int pass = 0; pass < nPasses; pass++) {
@@ -428,12 +563,22 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
     if (range > kRangeMax) range = kRangeMax;
     const int nPasses = (N + range - 1) / range;
     const size_t lds = (size_t)(range / 32 + range / 128) * sizeof(uint32_t);
+    const int smallGrid = (nRW + kBlock / 64 - 1) / (kBlock / 64);
+    if (W == 16)
+      hipLaunchKernelGGL(window_rank_small_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
+                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr);
+    else
+      hipLaunchKernelGGL(window_rank_small_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
+                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr);
+    F3S_HIP_CHECK(hipGetLastError());
     if (W == 16)
       hipLaunchKernelGGL(window_rank_kernel<16>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
-                         colIdx, N, range, nPasses, blockPartition, edgeToColumn, edgeToRow, hdr);
+                         colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,
+                         edgeToRow, hdr);
     else
       hipLaunchKernelGGL(window_rank_kernel<8>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
-                         colIdx, N, range, nPasses, blockPartition, edgeToColumn, edgeToRow, hdr);
+                         colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,
+                         edgeToRow, hdr);
     F3S_HIP_CHECK(hipGetLastError());
   }
   hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
