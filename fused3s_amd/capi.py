@@ -14,7 +14,8 @@ LIB_PATH = os.environ.get("F3S_AMD_LIB", os.path.join(_HERE, "libf3s_amd.so"))
 _lib = None
 
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
-           "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd"]
+           "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
+           "f3s_attention_workspace_bytes"]
 
 
 def lib():
@@ -36,8 +37,10 @@ def lib():
         L.f3s_preprocess_fill.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, ctypes.c_int64, vp, vp,
                                           vp, vp, vp, vp]
         L.f3s_attention_fwd.restype = ci
-        L.f3s_attention_fwd.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, vp, ctypes.c_float,
-                                        ci, vp, vp, vp]
+        L.f3s_attention_fwd.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, vp, vp, vp,
+                                        ctypes.c_float, ci, vp, vp, vp, cs, vp]
+        L.f3s_attention_workspace_bytes.restype = cs
+        L.f3s_attention_workspace_bytes.argtypes = [ci, ci]
         _lib = L
     return _lib
 
@@ -101,8 +104,14 @@ def preprocess(rowPtr, colIdx, N, H=16, W=16):
                 edgeToRow=edgeToRow)
 
 
+def attention_workspace(N, d, device):
+    """Scratch tensor for attention(..., workspace=...) (column-band schedule)."""
+    nbytes = lib().f3s_attention_workspace_bytes(N, d)
+    return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device)
+
+
 def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoftmax=True,
-              out=None):
+              out=None, workspace=None):
     """f3s_attention_fwd on the current stream; returns out fp32[N, d]."""
     L = lib()
     _dev(rwo, torch.int32, "rowWindowOffset")
@@ -129,7 +138,9 @@ def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoft
     if out is None:
         out = torch.empty((N, d), dtype=torch.float32, device=Q.device)
     with torch.cuda.device(Q.device):
-        _check(L.f3s_attention_fwd(_ptr(rwo), _ptr(order), _ptr(atox), _ptr(bitmap), N, d, dtype,
-                                   _ptr(Q), _ptr(K), _ptr(V), float(scalingFactor),
-                                   int(bool(applySoftmax)), _ptr(out), None, _stream()))
+        _check(L.f3s_attention_fwd(_ptr(rwo), _ptr(order), _ptr(atox), _ptr(bitmap), N,
+                                   atox.numel() // 16, d, dtype, _ptr(Q), _ptr(K), _ptr(V),
+                                   float(scalingFactor), int(bool(applySoftmax)), _ptr(out), None,
+                                   _ptr(workspace),
+                                   0 if workspace is None else workspace.numel(), _stream()))
     return out

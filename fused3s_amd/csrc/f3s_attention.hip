@@ -29,6 +29,9 @@
 // 938-945,1560-1561): running max starts at 0 and masked zeros take part in it, an unmasked
 // score that is exactly 0 is dropped like a masked one, the row sum uses un-rounded fp32
 // exponentials while P is rounded to fp16 for the second MFMA, empty rows give 0.
+#include <stdlib.h>
+#include <string.h>
+
 #include "f3s_common.h"
 
 namespace f3s {
@@ -366,9 +369,10 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
 }  // namespace
 
 int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
-                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
-                     int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
-                     int applySoftmax, float* out, unsigned long long* cuTimer,
+                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int64_t nTcb,
+                     int d, int dtype, const void* Q, const void* K, const void* V,
+                     float scalingFactor, int applySoftmax, float* out,
+                     unsigned long long* cuTimer, void* workspace, size_t wsBytes,
                      hipStream_t stream) {
   if (dtype != 0) return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16)", dtype);
   if (scalingFactor == 0.0f) return fail(-2, "f3s_attention_fwd: scalingFactor must be non-zero");
@@ -377,6 +381,21 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   // the reference divides unmasked scores by scalingFactor (src/F3S_kernel.cu:1666-1667);
   // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
+  // Experimental column-band schedule (f3s_attention_band.hip), opt-in with
+  // F3S_SCHEDULE=band in the environment plus a workspace: every wave walks the column range
+  // band by band so that K/V rows could be shared through L2. Measured on the 233k-node
+  // benchmark graph it is slower than the default (6.5 ms against 2.06 ms): waves owning heavy
+  // windows fall bands behind the others, the L2 hit rate stays at 45 %, and one wave per window
+  // leaves the long windows unsplit. It is kept, tested for correctness, as the base for a
+  // balanced version; the default is the workgroup-per-window kernel below.
+  static const bool bandSchedule = [] {
+    const char* e = getenv("F3S_SCHEDULE");
+    return e && strcmp(e, "band") == 0;
+  }();
+  const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
+  if (bandSchedule && workspace && !cuTimer && d <= 64 && nRW >= 2048 && nTcb >= 64 * nRW)
+    return launch_attention_band(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
+                                 V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
 #define F3S_DISPATCH(DD)                                                                       \
   case DD:                                                                                     \
     return applySoftmax ? launch_d<DD, true>(rowWindowOffset, windowOrder, sparseAToXidx,      \

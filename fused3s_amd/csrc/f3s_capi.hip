@@ -69,10 +69,17 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
                                      sparseAToXidx, tcbBitMap, static_cast<hipStream_t>(stream));
 }
 
+size_t f3s_attention_workspace_bytes(int N, int d) {
+  if (N < 0) N = 0;
+  if (d < 32) d = 32;
+  return f3s::attention_workspace_bytes(N, d);
+}
+
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
-                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int d,
-                      int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
-                      int applySoftmax, float* out, unsigned long long* cuTimer, void* stream) {
+                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int64_t nTCB,
+                      int d, int dtype, const void* Q, const void* K, const void* V,
+                      float scalingFactor, int applySoftmax, float* out,
+                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, void* stream) {
   if (N < 0) return f3s::fail(-2, "f3s_attention_fwd: negative N");
   if (N == 0) return 0;
   if (!rowWindowOffset || !Q || !K || !V || !out)
@@ -81,9 +88,14 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
       f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
       f3s::misaligned(tcbBitMap, 8))
     return f3s::fail(-1, "f3s_attention_fwd: Q/K/V/out/sparseAToXidx need 16-byte alignment");
-  return f3s::launch_attention(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, d,
+  if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd: negative nTCB");
+  if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
+    return f3s::fail(-1, "f3s_attention_fwd: null TC-block arrays");
+  if (workspace && f3s::misaligned(workspace, 4))
+    return f3s::fail(-1, "f3s_attention_fwd: workspace must be 4-byte aligned");
+  return f3s::launch_attention(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, nTCB, d,
                                dtype, Q, K, V, scalingFactor, applySoftmax, out, cuTimer,
-                               static_cast<hipStream_t>(stream));
+                               workspace, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

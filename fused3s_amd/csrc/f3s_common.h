@@ -22,10 +22,19 @@ int fail(int code, const char* fmt, ...);
 
 // attention (f3s_attention.hip)
 int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
-                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
-                     int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
-                     int applySoftmax, float* out, unsigned long long* cuTimer,
+                     const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int64_t nTcb,
+                     int d, int dtype, const void* Q, const void* K, const void* V,
+                     float scalingFactor, int applySoftmax, float* out,
+                     unsigned long long* cuTimer, void* workspace, size_t wsBytes,
                      hipStream_t stream);
+
+// column-band schedule (f3s_attention_band.hip)
+size_t attention_workspace_bytes(int N, int d);
+int launch_attention_band(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                          const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                          const void* Q, const void* K, const void* V, float scaleLog2,
+                          int applySoftmax, float* out, void* workspace, size_t wsBytes,
+                          hipStream_t stream);
 
 // preprocessing (f3s_preprocess.hip)
 size_t preprocess_workspace_bytes(int N, int E);

@@ -182,6 +182,9 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
     timer = torch::zeros({3 * nRW}, f32.dtype(torch::kInt64));
     timerPtr = reinterpret_cast<unsigned long long*>(timer.data_ptr());
   }
+  // scratch for the column-band schedule (used by the library only for dense graphs)
+  const size_t wsBytes = f3s_attention_workspace_bytes(nNodes, (int)d);
+  auto workspace = torch::empty({(int64_t)std::max<size_t>(wsBytes, 4)}, f32.dtype(torch::kUInt8));
   hipStream_t stream = at::hip::getCurrentHIPStream().stream();
   hipEvent_t start, stop;
   TORCH_CHECK(hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess);
@@ -189,8 +192,9 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
   const int rc = f3s_attention_fwd(
       rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,
       sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
-      nNodes, (int)d, F3S_DTYPE_F16, Q.data_ptr(), K.data_ptr(), V.data_ptr(), L.scalingFactor,
-      L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr, static_cast<void*>(stream));
+      nNodes, sparseAToXidx.numel() / 16, (int)d, F3S_DTYPE_F16, Q.data_ptr(), K.data_ptr(),
+      V.data_ptr(), L.scalingFactor, L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr,
+      workspace.data_ptr(), wsBytes, static_cast<void*>(stream));
   hipError_t e1 = hipEventRecord(stop, stream);
   hipError_t e2 = hipEventSynchronize(stop);
   float ms = 0.f;

@@ -93,7 +93,8 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *   rowWindowOffset [nRW+1], sparseAToXidx [nTCB*16], tcbBitMap [nTCB*4]   from preprocessing
  *   windowOrder [nRW] or NULL      launch order of the row windows: sortedRowWindows for the
  *                                  heavy-first schedule, NULL for natural order
- *   N, d                           nodes; head dimension (32, 64 or 128)
+ *   N, nTCB, d                     nodes; TC blocks (rowWindowOffset[nRW]); head dimension
+ *                                  (32, 64 or 128)
  *   dtype                          F3S_DTYPE_F16 (the reference's only type)
  *   Q, K, V [N*d]                  row-major, contiguous
  *   scalingFactor                  unmasked scores are DIVIDED by it (src/F3S_kernel.cu:1666-1667);
@@ -102,12 +103,27 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *   out [N*d] float                fully written (rows without edges get 0)
  *   cuTimer                        NULL, or 3*nRW uint64 {begin, end, cu id} per workgroup
  *                                  (the Clocked variants, src/F3S_kernel.cu:1178-1368, 1803-1997)
+ *   workspace, ws_bytes            NULL / 0, or device scratch of
+ *                                  f3s_attention_workspace_bytes(N, d) bytes (4-byte aligned).
+ *                                  Only the experimental column-band schedule uses it (selected
+ *                                  with F3S_SCHEDULE=band in the environment, for graphs with
+ *                                  >= 2048 windows and >= 64 TC blocks per window; results agree
+ *                                  with the default schedule within the tolerance of the
+ *                                  summation order).
  * Asynchronous on `stream`.
  */
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
-                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int d,
-                      int dtype, const void* Q, const void* K, const void* V, float scalingFactor,
-                      int applySoftmax, float* out, unsigned long long* cuTimer, void* stream);
+                      const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int64_t nTCB,
+                      int d, int dtype, const void* Q, const void* K, const void* V,
+                      float scalingFactor, int applySoftmax, float* out,
+                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, void* stream);
+
+/*
+ * Bytes of device scratch f3s_attention_fwd can use for a graph of N nodes at head dimension d
+ * (per-window block ranges of the column bands). The reference's launchers
+ * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
+ */
+size_t f3s_attention_workspace_bytes(int N, int d);
 
 #ifdef __cplusplus
 }

@@ -37,11 +37,11 @@ def test_argument_errors_are_statuses_not_exits():
     """Host-side argument checks run before any GPU work, so they are testable without a GPU."""
     from fused3s_amd import capi
     L = capi.lib()
-    rc = L.f3s_attention_fwd(None, None, None, None, -1, 64, 0, None, None, None, 1.0, 1, None,
-                             None, None)
+    rc = L.f3s_attention_fwd(None, None, None, None, -1, 0, 64, 0, None, None, None, 1.0, 1, None,
+                             None, None, 0, None)
     assert rc != 0 and b"negative" in L.f3s_last_error()
-    rc = L.f3s_attention_fwd(None, None, None, None, 5, 64, 0, None, None, None, 1.0, 1, None,
-                             None, None)
+    rc = L.f3s_attention_fwd(None, None, None, None, 5, 0, 64, 0, None, None, None, 1.0, 1, None,
+                             None, None, 0, None)
     assert rc != 0 and b"null" in L.f3s_last_error()
     n = ctypes.c_int64(0)
     rc = L.f3s_preprocess_count(None, None, 5, 0, 16, 16, None, None, None, None, None, None, 0,

@@ -3,6 +3,8 @@
 Tolerance (fp16 inputs, fp32 accumulation): max-abs 2e-2 and mean-relative 1e-3 against the
 reference-emulating oracle.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -18,15 +20,17 @@ def mean_rel(a, b):
     return float(np.abs(a - b).mean() / max(np.abs(b).mean(), 1e-30))
 
 
-def gpu_attention(pre, N, Q, K, V, scale, order=None, softmax=True):
+def gpu_attention(pre, N, Q, K, V, scale, order=None, softmax=True, band=False):
     from fused3s_amd import capi
     dev = "cuda"
     rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
     atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
     bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
     od = None if order is None else torch.as_tensor(np.asarray(order, np.int32)).to(dev)
+    ws = capi.attention_workspace(N, Q.shape[1], dev) if band else None
     out = capi.attention(rwo, od, atox, bm, N, torch.as_tensor(Q).to(dev),
-                         torch.as_tensor(K).to(dev), torch.as_tensor(V).to(dev), scale, softmax)
+                         torch.as_tensor(K).to(dev), torch.as_tensor(V).to(dev), scale, softmax,
+                         workspace=ws)
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -130,3 +134,37 @@ def test_end_to_end_hip_preprocess_then_attention(oracle_mod):
                                         V.numpy(), 8.0)
     got = out.cpu().numpy()
     assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL
+
+
+@pytest.mark.skipif(os.environ.get("F3S_SCHEDULE") != "band",
+                    reason="experimental column-band schedule: run with F3S_SCHEDULE=band")
+@pytest.mark.parametrize("d", [32, 64])
+def test_column_band_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
+    """A graph dense enough for the column-band schedule (>= 2048 windows, >= 64 TC blocks per
+    window): its result must match the reference-emulating oracle within the tolerance and the
+    workgroup-per-window kernel closely, for both window orders and without softmax."""
+    print("case band d=%d" % d, flush=True)
+    from fused3s_amd import synth
+    rp, ci = synth.make_graph("cfg3_chunglu_233k", scale=0.145)   # N = 33 779: N % 16 != 0
+    N = rp.numel() - 1
+    assert N % 16 != 0
+    rowPtr, colIdx = rp.numpy(), ci.numpy()
+    rng = np.random.default_rng(d)
+    Q, K, V = feats(rng, N, d)
+    scale = float(np.sqrt(d))
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    nRW = (N + 15) // 16
+    assert nRW >= 2048 and pre["blockCount"] >= 64 * nRW
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, Q, K, V, scale)
+    plain = gpu_attention(pre, N, Q, K, V, scale, pre["sortedRowWindows"])
+    for order in (pre["sortedRowWindows"], None):
+        got = gpu_attention(pre, N, Q, K, V, scale, order, band=True)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() < MAX_ABS
+        assert mean_rel(got, want) < MEAN_REL
+        assert np.abs(got - plain).max() < 2e-3
+    want_n = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                      pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
+    got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, band=True)
+    assert np.abs(got_n - want_n).max() < 2e-2 * max(1.0, np.abs(want_n).max())
