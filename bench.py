@@ -36,22 +36,32 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def host_bits(t):
+    """fp16 / bf16 device tensor -> numpy array the oracle takes (float16, or uint16 bits)."""
+    t = t.contiguous().cpu()
+    if t.dtype == torch.float16:
+        return t.numpy()
+    return t.view(torch.int16).numpy().view(np.uint16)
+
+
 def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
     """Time the CPU oracle (C + OpenMP restatement of textbook SDDMM/softmax/SpMM over CSR) on a
-    bounded sample: equally spaced slices of rows, grown until ~budget_s of CPU work is done."""
+    bounded sample: equally spaced slices of rows, grown until ~budget_s of CPU work is done.
+    Q, K, V: [N, d] of one head."""
     import oracle
     oracle.build()
     rp = rowPtr.cpu().numpy()
     ci = colIdx.cpu().numpy()
-    Qh, Kh, Vh = (x.cpu().numpy() for x in (Q, K, V))
+    dt = 0 if Q.dtype == torch.float16 else 1
+    Qh, Kh, Vh = (host_bits(x) for x in (Q, K, V))
     threads = oracle.num_threads()
     # calibrate on ~N/2048 evenly spaced rows, then size the sample for ~budget_s
     step = max(1, N // 512)
     t0 = time.time()
-    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, row_step=step)
+    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, dtype=dt, row_step=step)
     t_cal = time.time() - t0
     t0 = time.time()
-    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, rows=(0, 1))
+    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, dtype=dt, rows=(0, 1))
     t_fixed = time.time() - t0  # fp16 -> fp32 conversion of Q/K/V, paid by every call
     per_row = max(1e-9, (t_cal - t_fixed) / (N // step + 1))
     rows_target = int(min(N, max(64, budget_s / per_row)))
@@ -59,7 +69,7 @@ def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
     sel = np.arange(0, N, step)
     edges = int((rp[sel + 1] - rp[sel]).sum())
     t0 = time.time()
-    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, row_step=step)
+    oracle.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, dtype=dt, row_step=step)
     spent = time.time() - t0 - t_fixed
     rows_done = len(sel)
     tflops = 4.0 * d * edges / spent / 1e12 if spent > 0 else 0.0
@@ -109,9 +119,8 @@ def main():
     torch.cuda.set_device(dev)
     cfg = synth.CONFIGS[args.config]
     d = cfg["d"]
-    if cfg["dtype"] != "fp16" or cfg["heads"] != 1:
-        log("bench.py: config %s is not a single-head fp16 workload" % args.config)
-        sys.exit(2)
+    heads = cfg["heads"]
+    tdtype = torch.float16 if cfg["dtype"] == "fp16" else torch.bfloat16
 
     t0 = time.time()
     rowPtr, colIdx = synth.make_graph(args.config, seed=0, device=dev, scale=args.scale)
@@ -121,7 +130,11 @@ def main():
     deg = (rowPtr[1:] - rowPtr[:-1])
     log("graph %s: N=%d E=%d max_degree=%d (%.1f s to generate on the GPU)"
         % (args.config, N, E, int(deg.max()), time.time() - t0))
-    Q, K, V = synth.features(N, d, seed=0, device=dev)
+    # single head: [N, d] ~ N(0, 1); multi-head: [N, heads, d] ~ N(0, 1/d)
+    Q, K, V = synth.features(N, heads * d, seed=0, device=dev, dtype=tdtype,
+                             std=1.0 if heads == 1 else d ** -0.5)
+    if heads > 1:
+        Q, K, V = (x.view(N, heads, d) for x in (Q, K, V))
     scale = float(np.sqrt(d))
 
     # preprocessing (timed on its own; not part of the step)
@@ -149,12 +162,17 @@ def main():
         del src, dst
 
     order = None if args.natural_order else pre["sortedRowWindows"]
-    out = torch.empty((N, d), dtype=torch.float32, device=dev)
+    out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
     workspace = None if args.no_workspace else capi.attention_workspace(N, d, dev)
 
-    def step():
-        capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"], pre["tcbBitMap"], N,
-                       Q, K, V, scale, True, out=out, workspace=workspace)
+    if heads == 1:
+        def step():
+            capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"], pre["tcbBitMap"],
+                           N, Q, K, V, scale, True, out=out, workspace=workspace)
+    else:
+        def step():
+            capi.attention_heads(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
+                                 pre["tcbBitMap"], N, Q, K, V, scale, True, out=out)
 
     for _ in range(args.warmup):
         step()
@@ -172,23 +190,28 @@ def main():
     t_avg = float(kern_ms.mean()) * 1e-3
     t_med = float(np.median(kern_ms)) * 1e-3
 
-    f_eff = 4.0 * d * E
-    f_mfma = 1024.0 * d * nTCB
-    f_pad = 256.0 * (4 * d + 5) * nTCB
-    b_min = 3.0 * N * d * 2 + 4.0 * N * d + 96.0 * nTCB + 4.0 * (2 * nRW + 1)
-    b_gather = N * d * 2.0 + nTCB * (2 * 16 * d * 2.0 + 96) + 4.0 * N * d
+    D = heads * d  # all per-node byte and flop counts scale with the concatenated width
+    f_eff = 4.0 * D * E
+    f_mfma = 1024.0 * D * nTCB
+    f_pad = 256.0 * (4 * d + 5) * nTCB * heads
+    b_min = 3.0 * N * D * 2 + 4.0 * N * D + 96.0 * nTCB + 4.0 * (2 * nRW + 1)
+    b_gather = N * D * 2.0 + nTCB * (2 * 16 * D * 2.0 + 96.0 * heads) + 4.0 * N * D
     achieved = f_mfma / t_avg / 1e12
 
     result = {
-        "metric": "fused_3s_attention_effective_tflops_d%d_fp16" % d,
+        "metric": "fused_3s_attention_effective_tflops_d%d_%s%s"
+                  % (d, cfg["dtype"], "" if heads == 1 else "_%dheads" % heads),
         "value": f_eff / (wall / args.steps) / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "%s: N=%d E=%d d=%d fp16 single head, scalingFactor=sqrt(d), "
-                               "heavy-first window order" % (args.config, N, E, d),
+        "dtype": "f16" if cfg["dtype"] == "fp16" else "bf16", "data": "synthetic",
+        "config": {"workload": "%s: N=%d E=%d d=%d %s %s, scalingFactor=sqrt(d), %s window order"
+                               % (args.config, N, E, d, cfg["dtype"],
+                                  "single head" if heads == 1 else
+                                  "%d heads in one launch, output [N, %d]" % (heads, D),
+                                  "natural" if args.natural_order else "heavy-first"),
                    "nTCB": nTCB, "nRW": nRW, "max_tcb_per_window": int(cnt.max()),
                    "scale": args.scale},
         "kernel_ms_median": t_med * 1e3, "kernel_ms_mean": t_avg * 1e3,
@@ -203,8 +226,31 @@ def main():
     log("kernel: median %.3f ms  mean %.3f ms  effective %.1f TFLOP/s  MFMA %.1f TFLOP/s (%.1f%%)"
         % (t_med * 1e3, t_avg * 1e3, f_eff / t_med / 1e12, achieved,
            100 * achieved / PEAK_MFMA_F16_TFLOPS))
+    if heads > 1:
+        # the reference's way: one launch per head on contiguous per-head copies
+        per_head = [tuple(x[:, h].contiguous() for x in (Q, K, V)) for h in range(heads)]
+        outs = [torch.empty((N, d), dtype=torch.float32, device=dev) for _ in range(heads)]
+
+        def loop():
+            for h in range(heads):
+                capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
+                               pre["tcbBitMap"], N, *per_head[h], scale, True, out=outs[h])
+        loop()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        ev[0].record()
+        for i in range(args.steps):
+            loop()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        result["per_head_loop_ms_median"] = float(np.median(
+            [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]))
+        log("per-head loop of %d single-head launches: median %.3f ms"
+            % (heads, result["per_head_loop_ms_median"]))
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d,
+        # one head on the CPU; its rate in effective flops is the per-head rate of the whole job
+        q1, k1, v1 = (Q, K, V) if heads == 1 else (x[:, 0] for x in (Q, K, V))
+        result["cpu_baseline"] = cpu_baseline(rowPtr, colIdx, N, q1, k1, v1, scale, d,
                                               args.cpu_budget)
         log("cpu baseline:", result["cpu_baseline"])
     else:

@@ -15,7 +15,7 @@ _lib = None
 
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
            "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
-           "f3s_attention_workspace_bytes"]
+           "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads"]
 
 
 def lib():
@@ -41,6 +41,10 @@ def lib():
                                         ctypes.c_float, ci, vp, vp, vp, cs, vp]
         L.f3s_attention_workspace_bytes.restype = cs
         L.f3s_attention_workspace_bytes.argtypes = [ci, ci]
+        L.f3s_attention_fwd_heads.restype = ci
+        L.f3s_attention_fwd_heads.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, ci, vp,
+                                              vp, vp, ctypes.c_int64, ctypes.c_float, ci, vp,
+                                              ctypes.c_int64, vp]
         _lib = L
     return _lib
 
@@ -143,4 +147,49 @@ def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoft
                                    float(scalingFactor), int(bool(applySoftmax)), _ptr(out), None,
                                    _ptr(workspace),
                                    0 if workspace is None else workspace.numel(), _stream()))
+    return out
+
+
+def attention_heads(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoftmax=True,
+                    out=None):
+    """f3s_attention_fwd_heads on the current stream. Q, K, V: [N, nHeads, d] fp16 or bf16 whose
+    last two dimensions are contiguous (dim 0 may be pitched); returns out fp32[N, nHeads*d]."""
+    L = lib()
+    _dev(rwo, torch.int32, "rowWindowOffset")
+    _dev(atox, torch.int32, "sparseAToXidx")
+    _dev(bitmap, torch.uint64, "tcbBitMap")
+    if order is not None:
+        _dev(order, torch.int32, "windowOrder")
+        if order.numel() != rwo.numel() - 1:
+            raise RuntimeError("windowOrder must have one entry per row window")
+    if Q.dtype == torch.float16:
+        dtype = 0
+    elif Q.dtype == torch.bfloat16:
+        dtype = 1
+    else:
+        raise RuntimeError("Q/K/V must be float16 or bfloat16")
+    if Q.dim() != 3:
+        raise RuntimeError("Q/K/V must be [N, nHeads, d]")
+    nHeads, d = Q.shape[1], Q.shape[2]
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        if not t.is_cuda or t.dtype != Q.dtype or t.shape != Q.shape:
+            raise RuntimeError("%s must be a device tensor with Q's dtype and shape" % name)
+        if t.stride(2) != 1 or t.stride(1) != d or t.stride(0) != Q.stride(0):
+            raise RuntimeError("%s: heads must be contiguous inside a row, one row pitch for "
+                               "Q, K and V" % name)
+    if Q.shape[0] < N:
+        raise RuntimeError("Q/K/V have fewer than N rows")
+    if rwo.numel() != (N + 15) // 16 + 1:
+        raise RuntimeError("rowWindowOffset has %d entries, expected %d"
+                           % (rwo.numel(), (N + 15) // 16 + 1))
+    if out is None:
+        out = torch.empty((N, nHeads * d), dtype=torch.float32, device=Q.device)
+    elif out.dtype != torch.float32 or out.stride(1) != 1 or out.shape[1] != nHeads * d:
+        raise RuntimeError("out must be fp32 [N, nHeads*d] with contiguous rows")
+    with torch.cuda.device(Q.device):
+        _check(L.f3s_attention_fwd_heads(_ptr(rwo), _ptr(order), _ptr(atox), _ptr(bitmap), N,
+                                         atox.numel() // 16, nHeads, d, dtype, _ptr(Q), _ptr(K),
+                                         _ptr(V), Q.stride(0), float(scalingFactor),
+                                         int(bool(applySoftmax)), _ptr(out), out.stride(0),
+                                         _stream()))
     return out

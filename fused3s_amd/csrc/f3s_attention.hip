@@ -37,13 +37,27 @@
 namespace f3s {
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-template <int T>
-struct HalfVec {
-  typedef _Float16 type __attribute__((ext_vector_type(T)));
+// Vectors of the 16-bit input type ET (_Float16 or __bf16) and the MFMA that contracts them.
+template <typename ET, int L>
+struct Vec {
+  typedef ET type __attribute__((ext_vector_type(L)));
 };
+template <typename ET>
+__device__ __forceinline__ float4v mfma_16x16x32(typename Vec<ET, 8>::type a,
+                                                 typename Vec<ET, 8>::type b, float4v acc);
+template <>
+__device__ __forceinline__ float4v mfma_16x16x32<_Float16>(Vec<_Float16, 8>::type a,
+                                                           Vec<_Float16, 8>::type b,
+                                                           float4v acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ float4v mfma_16x16x32<__bf16>(Vec<__bf16, 8>::type a,
+                                                         Vec<__bf16, 8>::type b, float4v acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -62,10 +76,10 @@ __device__ __forceinline__ float row_sum4(float v) {
 }
 
 // Everything one TC-block pair needs from memory, as it sits in registers.
-template <int D>
+template <typename ET, int D>
 struct PairData {
-  half8 kA[D / 32], kB[D / 32];            // K rows of the two blocks (A operand of S^T)
-  typename HalfVec<D / 16>::type vv[8];    // V pieces of this lane's 8 contraction slots
+  typename Vec<ET, 8>::type kA[D / 32], kB[D / 32];  // K rows of the two blocks (A operand of S^T)
+  typename Vec<ET, D / 16>::type vv[8];    // V pieces of this lane's 8 contraction slots
   unsigned maskA, maskB;                   // bitmap byte holding this lane's 4 bits per block
 };
 // Metadata of a pair, one dword per lane from a single load: lanes 0..31 hold the 32 column ids
@@ -94,27 +108,43 @@ __device__ __forceinline__ unsigned cu_key() {
   return ((xcc & 0xFu) << 8) | ((hw >> 8) & 0xFFu);
 }
 
-template <int D, int NWAVES, bool SOFTMAX, bool CLOCKED>
+// HEADS = false: Q/K/V are [N, D] contiguous, one workgroup per window (blockIdx.x = position in
+// the window order). HEADS = true: Q/K/V are [N, nHeads, D] with a row pitch of ldIn elements,
+// out is [N, nHeads * D] with a row pitch of ldOut floats, and blockIdx.x = position * nHeads +
+// head, so that the workgroups of one window's heads are dispatched together and share the
+// window's column ids and bitmaps (and the neighbouring pieces of its K/V rows) in L2.
+template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS>
 __global__ __launch_bounds__(NWAVES * 64)
 __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
-    int nRW, const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
-    const _Float16* __restrict__ V, float scaleLog2, float* __restrict__ out,
-    unsigned long long* __restrict__ cuTimer) {
+    int nRW, const ET* __restrict__ Q, const ET* __restrict__ K, const ET* __restrict__ V,
+    float scaleLog2, float* __restrict__ out, unsigned long long* __restrict__ cuTimer,
+    int nHeads, int ldIn, int ldOut) {
+  typedef typename Vec<ET, 8>::type half8;
   constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
   unsigned long long tBegin = 0;
   if constexpr (CLOCKED) tBegin = realtime_ticks();
   constexpr int KS = D / 32;  // MFMA k-steps of the score product
   constexpr int OSTRIDE = D + 4;
-  typedef typename HalfVec<T>::type vrow_t;
+  typedef typename Vec<ET, T>::type vrow_t;
 
   __shared__ float sM[NWAVES][16];
   __shared__ float sL[NWAVES][16];
   __shared__ __align__(16) float sO[NWAVES][16][OSTRIDE];
 
-  const int w = windowOrder ? windowOrder[blockIdx.x] : (int)blockIdx.x;
+  const int pos = HEADS ? (int)(blockIdx.x / (unsigned)nHeads) : (int)blockIdx.x;
+  const int head = HEADS ? (int)(blockIdx.x - (unsigned)pos * (unsigned)nHeads) : 0;
+  const int w = windowOrder ? windowOrder[pos] : pos;
   if ((unsigned)w >= (unsigned)nRW) return;  // a corrupt order entry must not index out of range
+  // row pitches in elements / bytes; compile-time constants for the single-head layout
+  const int pitchIn = HEADS ? ldIn : D;
+  const int pitchOut = HEADS ? ldOut : D;
+  const uint32_t rowBytes = (uint32_t)pitchIn * 2u;
+  Q += head * D;
+  K += head * D;
+  V += head * D;
+  out += head * D;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int g = lane >> 4;
@@ -125,16 +155,18 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   const int nPairs = (t1 - t0 + 1) >> 1;
 
   // B operand of the score product: this lane's query row, features 32i + 8g .. +7
+  typedef int int4v __attribute__((ext_vector_type(4)));
+  const int4v zero16 = {0, 0, 0, 0};
   half8 qf[KS];
   {
     const int64_t qrow = (int64_t)w * 16 + c;
     if (qrow < N) {
-      const half8* qp = reinterpret_cast<const half8*>(Q + qrow * D) + g;
+      const half8* qp = reinterpret_cast<const half8*>(Q + qrow * pitchIn) + g;
 #pragma unroll
       for (int i = 0; i < KS; i++) qf[i] = qp[4 * i];
     } else {
 #pragma unroll
-      for (int i = 0; i < KS; i++) qf[i] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+      for (int i = 0; i < KS; i++) qf[i] = __builtin_bit_cast(half8, zero16);
     }
   }
 
@@ -165,9 +197,13 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   };
   auto lane_read = [&](int v, int srcLane) { return __builtin_amdgcn_ds_bpermute(srcLane * 4, v); };
   auto load_data = [&](const PairIndex& ix) {
-    PairData<D> pd;
-    // 32-bit byte offsets from the uniform K / V bases (the launcher checks N*D*2 < 4 GiB): one
-    // address register per gathered row instead of a 64-bit pointer per load
+    PairData<ET, D> pd;
+    // 32-bit byte offsets from the uniform K / V bases (the launcher checks that K and V span
+    // less than 4 GiB, and N < 2^24 for the pitched layout, whose row offset is a 24-bit
+    // multiply): one address register per gathered row instead of a 64-bit pointer per load
+    auto row_offset = [&](uint32_t row) {
+      return HEADS ? __umul24(row, rowBytes) : row * (uint32_t)(D * 2);
+    };
     const char* Kb = reinterpret_cast<const char*>(K);
     const char* Vb = reinterpret_cast<const char*>(V);
     // K is fetched with four adjacent lanes on one 64-byte piece of a row (lane -> slot lane/4,
@@ -175,8 +211,8 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     // pieces to the MFMA layout (slot c, chunk g) with a cross-lane permute.
     const uint32_t kRowA = (uint32_t)lane_read(ix.meta, lane >> 2);
     const uint32_t kRowB = (uint32_t)lane_read(ix.meta, 16 + (lane >> 2));
-    const uint32_t koA = kRowA * (uint32_t)(D * 2) + (uint32_t)((lane & 3) * 16);
-    const uint32_t koB = kRowB * (uint32_t)(D * 2) + (uint32_t)((lane & 3) * 16);
+    const uint32_t koA = row_offset(kRowA) + (uint32_t)((lane & 3) * 16);
+    const uint32_t koB = row_offset(kRowB) + (uint32_t)((lane & 3) * 16);
 #pragma unroll
     for (int i = 0; i < KS; i++) {
       pd.kA[i] = *reinterpret_cast<const half8*>(Kb + koA + 64 * i);
@@ -185,7 +221,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
 #pragma unroll
     for (int k = 0; k < 8; k++) {
       const uint32_t vRow = (uint32_t)lane_read(ix.meta, (k < 4 ? 0 : 16) + 4 * g + (k & 3));
-      const uint32_t vo = vRow * (uint32_t)(D * 2) + (uint32_t)(c * T * 2);
+      const uint32_t vo = row_offset(vRow) + (uint32_t)(c * T * 2);
       pd.vv[k] = *reinterpret_cast<const vrow_t*>(Vb + vo);
     }
     pd.maskA = ((unsigned)lane_read(ix.meta, 32 + (maskByte >> 2)) >> (8 * (maskByte & 3))) & 0xFFu;
@@ -195,21 +231,20 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   // lane (g, c) takes the 16 bytes that lane 4c + g loaded
   const int permAddr = (4 * c + g) * 4;
   auto to_mfma_layout = [&](half8 v) {
-    typedef int int4v __attribute__((ext_vector_type(4)));
     int4v x = __builtin_bit_cast(int4v, v);
 #pragma unroll
     for (int k = 0; k < 4; k++) x[k] = __builtin_amdgcn_ds_bpermute(permAddr, x[k]);
     return __builtin_bit_cast(half8, x);
   };
-  auto compute = [&](const PairData<D>& pd, int p) {
+  auto compute = [&](const PairData<ET, D>& pd, int p) {
     const bool hasB = (t0 + 2 * p + 1) < t1;
     const unsigned bitsA = (pd.maskA >> maskShift) & 0xFu;
     const unsigned bitsB = hasB ? ((pd.maskB >> maskShift) & 0xFu) : 0u;
     float4v sA = {0.f, 0.f, 0.f, 0.f}, sB = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < KS; i++) {
-      sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_mfma_layout(pd.kA[i]), qf[i], sA, 0, 0, 0);
-      sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_mfma_layout(pd.kB[i]), qf[i], sB, 0, 0, 0);
+      sA = mfma_16x16x32<ET>(to_mfma_layout(pd.kA[i]), qf[i], sA);
+      sB = mfma_16x16x32<ET>(to_mfma_layout(pd.kB[i]), qf[i], sB);
     }
     float s[8];
 #pragma unroll
@@ -233,21 +268,21 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
       for (int i = 0; i < 8; i++) {
         const float e = (s[i] == 0.0f) ? 0.0f : fast_exp2(s[i] - mx);
         sum += e;
-        pf[i] = (_Float16)e;
+        pf[i] = (ET)e;
       }
       l = fmaf(alpha, l, sum);
 #pragma unroll
       for (int j = 0; j < T; j++) o[j] *= alpha;
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; i++) pf[i] = (_Float16)s[i];
+      for (int i = 0; i < 8; i++) pf[i] = (ET)s[i];
     }
 #pragma unroll
     for (int j = 0; j < T; j++) {
       half8 va;
 #pragma unroll
       for (int k = 0; k < 8; k++) va[k] = pd.vv[k][j];
-      o[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pf, o[j], 0, 0, 0);
+      o[j] = mfma_16x16x32<ET>(va, pf, o[j]);
     }
   };
 
@@ -265,7 +300,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     PairIndex m0 = load_index(p);
     PairIndex m1 = load_index(clamp_pair(p + NWAVES));
     PairIndex m2 = load_index(clamp_pair(p + 2 * NWAVES));
-    PairData<D> pd0 = load_data(m0), pd1, pd2;
+    PairData<ET, D> pd0 = load_data(m0), pd1, pd2;
     m0 = load_index(clamp_pair(p + 3 * NWAVES));
     pd1 = load_data(m1);
 #define F3S_STEP(CUR, FILL, MUSE, MFILL)              \
@@ -331,7 +366,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
         acc.w += ov.w;
       }
     }
-    *reinterpret_cast<float4*>(out + row * D + cv * 4) = acc;
+    *reinterpret_cast<float4*>(out + row * pitchOut + cv * 4) = acc;
   }
   if constexpr (CLOCKED) {
     // {first tick, last tick, CU} of this workgroup, as the reference's timed kernels record
@@ -345,25 +380,60 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   }
 }
 
-template <int D, bool SOFTMAX>
+struct HeadLayout {
+  int nHeads;  // 0: contiguous [N, d] single head
+  int ldIn;    // row pitch of Q/K/V in elements
+  int ldOut;   // row pitch of out in floats
+};
+
+template <typename ET, int D, bool SOFTMAX>
 int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, const uint64_t* bitmap,
              int N, const void* Q, const void* K, const void* V, float scaleLog2, float* out,
-             unsigned long long* cuTimer, hipStream_t stream) {
+             unsigned long long* cuTimer, HeadLayout hl, hipStream_t stream) {
   constexpr int NWAVES = 4;
   const int nRW = (N + kWinRows - 1) / kWinRows;
   if (nRW == 0) return 0;
   const auto* bm = reinterpret_cast<const uint8_t*>(bitmap);
-  const auto* q = static_cast<const _Float16*>(Q);
-  const auto* k = static_cast<const _Float16*>(K);
-  const auto* v = static_cast<const _Float16*>(V);
-  if (cuTimer)
-    hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX, true>), dim3(nRW), dim3(NWAVES * 64), 0,
-                       stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer);
+  const auto* q = static_cast<const ET*>(Q);
+  const auto* k = static_cast<const ET*>(K);
+  const auto* v = static_cast<const ET*>(V);
+  const dim3 block(NWAVES * 64);
+  if (hl.nHeads > 0)
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, true>),
+                       dim3((unsigned)nRW * (unsigned)hl.nHeads), block, 0, stream, rwo, order,
+                       atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer, hl.nHeads, hl.ldIn,
+                       hl.ldOut);
+  else if (cuTimer)
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, true, false>), dim3(nRW), block, 0,
+                       stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer, 1,
+                       D, D);
   else
-    hipLaunchKernelGGL((f3s_fwd_kernel<D, NWAVES, SOFTMAX, false>), dim3(nRW), dim3(NWAVES * 64),
-                       0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer);
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false>), dim3(nRW), block,
+                       0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer,
+                       1, D, D);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
+}
+
+template <typename ET>
+int dispatch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox,
+               const uint64_t* bitmap, int N, int d, const void* Q, const void* K, const void* V,
+               float scaleLog2, int applySoftmax, float* out, unsigned long long* cuTimer,
+               HeadLayout hl, hipStream_t stream) {
+#define F3S_DISPATCH(DD)                                                                        \
+  case DD:                                                                                      \
+    return applySoftmax ? launch_d<ET, DD, true>(rwo, order, atox, bitmap, N, Q, K, V,          \
+                                                 scaleLog2, out, cuTimer, hl, stream)           \
+                        : launch_d<ET, DD, false>(rwo, order, atox, bitmap, N, Q, K, V,         \
+                                                  scaleLog2, out, cuTimer, hl, stream);
+  switch (d) {
+    F3S_DISPATCH(32)
+    F3S_DISPATCH(64)
+    F3S_DISPATCH(128)
+    default:
+      return fail(-2, "f3s_attention_fwd: head dim %d unsupported (32, 64, 128)", d);
+  }
+#undef F3S_DISPATCH
 }
 
 }  // namespace
@@ -374,7 +444,8 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                      float scalingFactor, int applySoftmax, float* out,
                      unsigned long long* cuTimer, void* workspace, size_t wsBytes,
                      hipStream_t stream) {
-  if (dtype != 0) return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16)", dtype);
+  if (dtype != 0 && dtype != 1)
+    return fail(-3, "f3s_attention_fwd: dtype %d not supported (0 = fp16, 1 = bf16)", dtype);
   if (scalingFactor == 0.0f) return fail(-2, "f3s_attention_fwd: scalingFactor must be non-zero");
   if ((int64_t)N * d * 2 >= (int64_t)1 << 32)
     return fail(-2, "f3s_attention_fwd: K and V must each be smaller than 4 GiB (N*d*2 bytes)");
@@ -393,25 +464,49 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
     return e && strcmp(e, "band") == 0;
   }();
   const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
-  if (bandSchedule && workspace && !cuTimer && d <= 64 && nRW >= 2048 && nTcb >= 64 * nRW)
+  if (bandSchedule && dtype == 0 && workspace && !cuTimer && d <= 64 && nRW >= 2048 && nTcb >= 64 * nRW)
     return launch_attention_band(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
                                  V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
-#define F3S_DISPATCH(DD)                                                                       \
-  case DD:                                                                                     \
-    return applySoftmax ? launch_d<DD, true>(rowWindowOffset, windowOrder, sparseAToXidx,      \
-                                             bitmap, N, Q, K, V, scaleLog2, out, cuTimer,      \
-                                             stream)                                           \
-                        : launch_d<DD, false>(rowWindowOffset, windowOrder, sparseAToXidx,     \
-                                              bitmap, N, Q, K, V, scaleLog2, out, cuTimer,     \
-                                              stream);
-  switch (d) {
-    F3S_DISPATCH(32)
-    F3S_DISPATCH(64)
-    F3S_DISPATCH(128)
-    default:
-      return fail(-2, "f3s_attention_fwd: head dim %d unsupported (32, 64, 128)", d);
-  }
-#undef F3S_DISPATCH
+  const HeadLayout single = {0, d, d};
+  return dtype == 0 ? dispatch_d<_Float16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N,
+                                           d, Q, K, V, scaleLog2, applySoftmax, out, cuTimer,
+                                           single, stream)
+                    : dispatch_d<__bf16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d,
+                                         Q, K, V, scaleLog2, applySoftmax, out, cuTimer, single,
+                                         stream);
+}
+
+int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                           const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
+                           int nHeads, int d, int dtype, const void* Q, const void* K,
+                           const void* V, int64_t ldIn, float scalingFactor, int applySoftmax,
+                           float* out, int64_t ldOut, hipStream_t stream) {
+  if (dtype != 0 && dtype != 1)
+    return fail(-3, "f3s_attention_fwd_heads: dtype %d not supported (0 = fp16, 1 = bf16)", dtype);
+  if (scalingFactor == 0.0f)
+    return fail(-2, "f3s_attention_fwd_heads: scalingFactor must be non-zero");
+  if (nHeads < 1 || nHeads > 1024)
+    return fail(-2, "f3s_attention_fwd_heads: nHeads %d out of range (1..1024)", nHeads);
+  if (ldIn < (int64_t)nHeads * d || ldOut < (int64_t)nHeads * d)
+    return fail(-2, "f3s_attention_fwd_heads: row pitches must be at least nHeads*d");
+  if (ldIn % 8 != 0 || ldOut % 4 != 0)
+    return fail(-2, "f3s_attention_fwd_heads: rows must stay 16-byte aligned (ldIn %% 8 == 0, "
+                    "ldOut %% 4 == 0)");
+  if (ldIn * 2 >= ((int64_t)1 << 24) || N >= (1 << 24))
+    return fail(-2, "f3s_attention_fwd_heads: N and the row pitch in bytes must be below 2^24");
+  if ((int64_t)N * ldIn * 2 >= (int64_t)1 << 32)
+    return fail(-2, "f3s_attention_fwd_heads: K and V must each span less than 4 GiB");
+  const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
+  if (nRW * nHeads >= ((int64_t)1 << 31))
+    return fail(-2, "f3s_attention_fwd_heads: too many (window, head) workgroups");
+  const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
+  const HeadLayout hl = {nHeads, (int)ldIn, (int)ldOut};
+  return dtype == 0 ? dispatch_d<_Float16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N,
+                                           d, Q, K, V, scaleLog2, applySoftmax, out, nullptr, hl,
+                                           stream)
+                    : dispatch_d<__bf16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d,
+                                         Q, K, V, scaleLog2, applySoftmax, out, nullptr, hl,
+                                         stream);
 }
 
 }  // namespace f3s

@@ -98,4 +98,25 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
                                workspace, ws_bytes, static_cast<hipStream_t>(stream));
 }
 
+int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                            const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
+                            int64_t nTCB, int nHeads, int d, int dtype, const void* Q,
+                            const void* K, const void* V, int64_t ldIn, float scalingFactor,
+                            int applySoftmax, float* out, int64_t ldOut, void* stream) {
+  if (N < 0) return f3s::fail(-2, "f3s_attention_fwd_heads: negative N");
+  if (N == 0) return 0;
+  if (!rowWindowOffset || !Q || !K || !V || !out)
+    return f3s::fail(-1, "f3s_attention_fwd_heads: null pointer");
+  if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
+      f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
+      f3s::misaligned(tcbBitMap, 8))
+    return f3s::fail(-1, "f3s_attention_fwd_heads: Q/K/V/out/sparseAToXidx need 16-byte alignment");
+  if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd_heads: negative nTCB");
+  if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
+    return f3s::fail(-1, "f3s_attention_fwd_heads: null TC-block arrays");
+  return f3s::launch_attention_heads(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N,
+                                     nHeads, d, dtype, Q, K, V, ldIn, scalingFactor, applySoftmax,
+                                     out, ldOut, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

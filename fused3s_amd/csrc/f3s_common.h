@@ -28,6 +28,12 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                      unsigned long long* cuTimer, void* workspace, size_t wsBytes,
                      hipStream_t stream);
 
+int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                           const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
+                           int nHeads, int d, int dtype, const void* Q, const void* K,
+                           const void* V, int64_t ldIn, float scalingFactor, int applySoftmax,
+                           float* out, int64_t ldOut, hipStream_t stream);
+
 // column-band schedule (f3s_attention_band.hip)
 size_t attention_workspace_bytes(int N, int d);
 int launch_attention_band(const int32_t* rowWindowOffset, const int32_t* windowOrder,

@@ -129,6 +129,27 @@ void write_cu_time(const torch::Tensor& timer, int64_t nBlocks, const std::strin
     out << (double)kv.second.first / 1e5 << " " << (double)kv.second.second / 1e5 << std::endl;
 }
 
+// Runs `launch(stream)` on PyTorch's current stream between two events, blocks on the stop event
+// like the reference's launchers (src/F3S_kernel.cu:436-451) and returns the elapsed ms.
+template <typename F>
+float timed_launch(const char* what, F&& launch) {
+  hipStream_t stream = at::hip::getCurrentHIPStream().stream();
+  hipEvent_t start, stop;
+  TORCH_CHECK(hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess);
+  TORCH_CHECK(hipEventRecord(start, stream) == hipSuccess);
+  const int rc = launch(static_cast<void*>(stream));
+  hipError_t e1 = hipEventRecord(stop, stream);
+  hipError_t e2 = hipEventSynchronize(stop);
+  float ms = 0.f;
+  hipError_t e3 = hipEventElapsedTime(&ms, start, stop);
+  (void)hipEventDestroy(start);
+  (void)hipEventDestroy(stop);
+  check_status(rc, what);
+  TORCH_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "HIP event timing failed: ",
+              hipGetErrorString(e2 != hipSuccess ? e2 : (e1 != hipSuccess ? e1 : e3)));
+  return ms;
+}
+
 struct Launch {
   const torch::Tensor* order;  // nullptr = natural window order
   float scalingFactor;
@@ -147,9 +168,9 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
                                       const torch::Tensor& Q, const torch::Tensor& K,
                                       const torch::Tensor& V, int nWarpPerBlock, const Launch& L) {
   TORCH_CHECK(Q.dim() == 2 && K.dim() == 2 && V.dim() == 2, "Q, K, V must be [N, d]");
-  TORCH_CHECK(Q.scalar_type() == torch::kHalf && K.scalar_type() == torch::kHalf &&
-                  V.scalar_type() == torch::kHalf,
-              "Q, K, V must be float16");
+  TORCH_CHECK((Q.scalar_type() == torch::kHalf || Q.scalar_type() == torch::kBFloat16) &&
+                  K.scalar_type() == Q.scalar_type() && V.scalar_type() == Q.scalar_type(),
+              "Q, K, V must all be float16 (the reference's type) or all bfloat16");
   TORCH_CHECK(Q.is_cuda() && K.is_cuda() && V.is_cuda() && rowWindowOffset.is_cuda() &&
                   sparseAToXidx.is_cuda() && tcbBitMap.is_cuda(),
               "all tensors must be CUDA tensors");
@@ -182,31 +203,67 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
     timer = torch::zeros({3 * nRW}, f32.dtype(torch::kInt64));
     timerPtr = reinterpret_cast<unsigned long long*>(timer.data_ptr());
   }
-  // scratch for the column-band schedule (used by the library only for dense graphs)
+  // scratch of the opt-in column-band schedule (F3S_SCHEDULE=band); unused otherwise
   const size_t wsBytes = f3s_attention_workspace_bytes(nNodes, (int)d);
   auto workspace = torch::empty({(int64_t)std::max<size_t>(wsBytes, 4)}, f32.dtype(torch::kUInt8));
-  hipStream_t stream = at::hip::getCurrentHIPStream().stream();
-  hipEvent_t start, stop;
-  TORCH_CHECK(hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess);
-  TORCH_CHECK(hipEventRecord(start, stream) == hipSuccess);
-  const int rc = f3s_attention_fwd(
-      rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,
-      sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
-      nNodes, sparseAToXidx.numel() / 16, (int)d, F3S_DTYPE_F16, Q.data_ptr(), K.data_ptr(),
-      V.data_ptr(), L.scalingFactor, L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr,
-      workspace.data_ptr(), wsBytes, static_cast<void*>(stream));
-  hipError_t e1 = hipEventRecord(stop, stream);
-  hipError_t e2 = hipEventSynchronize(stop);
-  float ms = 0.f;
-  hipError_t e3 = hipEventElapsedTime(&ms, start, stop);
-  (void)hipEventDestroy(start);
-  (void)hipEventDestroy(stop);
-  check_status(rc, "f3s_attention_fwd");
-  TORCH_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "HIP event timing failed: ",
-              hipGetErrorString(e2 != hipSuccess ? e2 : (e1 != hipSuccess ? e1 : e3)));
+  const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
+  const float ms = timed_launch("f3s_attention_fwd", [&](void* stream) {
+    return f3s_attention_fwd(
+        rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,
+        sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
+        nNodes, sparseAToXidx.numel() / 16, (int)d, dtype, Q.data_ptr(), K.data_ptr(),
+        V.data_ptr(), L.scalingFactor, L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr,
+        workspace.data_ptr(), wsBytes, stream);
+  });
   if (L.timerFile) write_cu_time(timer, nRW, L.timerFile);
   auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));
   return {time, out, sddmmResult};
+}
+
+// Multi-head call, beyond the reference's surface: its graph-transformer callers run
+// f3s_1tb1rw_scheduled_permuteV_scaleQK (src/F3S.cpp:247-270) once per head and concatenate.
+// Q, K, V are [N, nHeads, d] (heads contiguous inside a row, rows may be pitched), fp16 or bf16;
+// returns {time_ms, out fp32[N, nHeads*d], empty} from ONE launch over all (window, head) pairs.
+std::vector<torch::Tensor> f3sMultiHeadScaleQK(torch::Tensor rowWindowOffset,
+                                               torch::Tensor sortedRowWindows,
+                                               torch::Tensor sparseAToXidx,
+                                               torch::Tensor tcbBitMap, int nNodes,
+                                               torch::Tensor Q, torch::Tensor K, torch::Tensor V,
+                                               float scalingFactor) {
+  TORCH_CHECK(Q.dim() == 3 && K.sizes() == Q.sizes() && V.sizes() == Q.sizes(),
+              "Q, K, V must be [N, nHeads, d] with identical shapes");
+  TORCH_CHECK((Q.scalar_type() == torch::kHalf || Q.scalar_type() == torch::kBFloat16) &&
+                  K.scalar_type() == Q.scalar_type() && V.scalar_type() == Q.scalar_type(),
+              "Q, K, V must all be float16 or all bfloat16");
+  const int64_t nHeads = Q.size(1), d = Q.size(2);
+  for (const torch::Tensor* t : {&Q, &K, &V})
+    TORCH_CHECK(t->is_cuda() && t->stride(2) == 1 && t->stride(1) == d &&
+                    t->stride(0) == Q.stride(0),
+                "Q, K, V must be CUDA tensors with heads contiguous inside a row and one row "
+                "pitch");
+  for (const torch::Tensor* t : {&rowWindowOffset, &sortedRowWindows, &sparseAToXidx, &tcbBitMap})
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous(), "TC-block tensors must be contiguous CUDA "
+                                                    "tensors");
+  TORCH_CHECK(Q.size(0) >= nNodes, "Q, K, V need at least nNodes rows");
+  const int64_t nRW = rowWindowOffset.numel() - 1;
+  TORCH_CHECK(nRW == ((int64_t)nNodes + 15) / 16,
+              "rowWindowOffset does not match nNodes (expected ceil(nNodes/16)+1 entries)");
+  TORCH_CHECK(sortedRowWindows.numel() == nRW && sortedRowWindows.scalar_type() == torch::kInt32,
+              "sortedRowWindows must be int32 with one entry per window");
+  c10::DeviceGuard guard(Q.device());
+  auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(Q.device());
+  auto out = torch::empty({(int64_t)nNodes, nHeads * d}, f32);
+  const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
+  const float ms = timed_launch("f3s_attention_fwd_heads", [&](void* stream) {
+    return f3s_attention_fwd_heads(
+        rowWindowOffset.data_ptr<int>(), sortedRowWindows.data_ptr<int>(),
+        sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
+        nNodes, sparseAToXidx.numel() / 16, (int)nHeads, (int)d, dtype, Q.data_ptr(),
+        K.data_ptr(), V.data_ptr(), Q.stride(0), scalingFactor, 1, out.data_ptr<float>(),
+        out.stride(0), stream);
+  });
+  auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));
+  return {time, out, torch::zeros({0}, f32)};
 }
 
 // F3S.f3s_1tb1rw (src/F3S.cpp:145-183)
@@ -291,4 +348,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "fused3S 1tb1rw scheduled permuteV");
   m.def("f3s_1tb1rw_scheduled_permuteV_scaleQK", &f3s1tb1rwScheduledPermuteVScaleQK,
         "fused3S 1tb1rw scheduled permuteV scaleQK");
+  m.def("f3s_multihead_scaleQK", &f3sMultiHeadScaleQK,
+        "fused3S over [N, heads, d] Q/K/V in one launch (fp16 or bf16), heavy-first order");
 }

@@ -95,7 +95,8 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *                                  heavy-first schedule, NULL for natural order
  *   N, nTCB, d                     nodes; TC blocks (rowWindowOffset[nRW]); head dimension
  *                                  (32, 64 or 128)
- *   dtype                          F3S_DTYPE_F16 (the reference's only type)
+ *   dtype                          F3S_DTYPE_F16 (the reference's only type) or F3S_DTYPE_BF16
+ *                                  (bf16 MFMA; the probabilities are then rounded to bf16)
  *   Q, K, V [N*d]                  row-major, contiguous
  *   scalingFactor                  unmasked scores are DIVIDED by it (src/F3S_kernel.cu:1666-1667);
  *                                  1.0 = unscaled (:612-613)
@@ -124,6 +125,22 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
  * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);
+
+/*
+ * The same fused kernel over nHeads attention heads in one launch: Q, K, V are [N, nHeads, d]
+ * with a row pitch of ldIn elements (head h of node i starts at element i*ldIn + h*d), out is
+ * [N, nHeads*d] fp32 with a row pitch of ldOut floats, i.e. the per-head results already
+ * concatenated. All heads share one graph (one TC-block structure). The reference has no
+ * multi-head entry: its callers run f3s_1tb1rw_scheduled_permuteV_scaleQK (src/F3S.cpp:247-270)
+ * once per head on contiguous per-head copies and concatenate; this call returns what that loop
+ * returns. ldIn % 8 == 0, ldOut % 4 == 0, N < 2^24, ldIn*2 < 2^24, N*ldIn*2 < 2^32.
+ * Asynchronous on `stream`.
+ */
+int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                            const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
+                            int64_t nTCB, int nHeads, int d, int dtype, const void* Q,
+                            const void* K, const void* V, int64_t ldIn, float scalingFactor,
+                            int applySoftmax, float* out, int64_t ldOut, void* stream);
 
 #ifdef __cplusplus
 }

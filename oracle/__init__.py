@@ -55,6 +55,8 @@ def lib():
         L.f3s_oracle_half_to_float.argtypes = [ctypes.c_uint16]
         L.f3s_oracle_round_to_half.restype = ctypes.c_float
         L.f3s_oracle_round_to_half.argtypes = [ctypes.c_float]
+        L.f3s_oracle_round_to_bf16.argtypes = [ctypes.c_float]
+        L.f3s_oracle_round_to_bf16.restype = ctypes.c_float
         L.f3s_oracle_num_threads.restype = ci
         _lib = L
     return _lib

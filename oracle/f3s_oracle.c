@@ -110,6 +110,16 @@ static float bf16_bits_to_float(uint16_t b) {
   return f;
 }
 
+/* fp32 -> bf16 -> fp32, round to nearest even (finite inputs) */
+static float round_to_bf16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  x += 0x7FFFu + ((x >> 16) & 1u);
+  x &= 0xFFFF0000u;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
 static float *to_float(const uint16_t *src, int64_t n, int dtype) {
   float *dst = (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
   if (!dst) return NULL;
@@ -124,6 +134,7 @@ static float *to_float(const uint16_t *src, int64_t n, int dtype) {
 /* exported so tests can pin the conversions against numpy.float16 */
 float f3s_oracle_half_to_float(uint16_t h) { return half_bits_to_float(h); }
 float f3s_oracle_round_to_half(float f) { return round_to_half(f); }
+float f3s_oracle_round_to_bf16(float f) { return round_to_bf16(f); }
 
 /* ------------------------------------------------------------ preprocessing */
 
@@ -327,7 +338,7 @@ static inline int tcb_bit(const uint64_t *bitmap, int64_t t, int rl, int cl) {
  * sortedRowWindows argument of the reference is not needed here.
  * Rows >= N of the last window are treated as all-zero Q and never written.
  * dtype: 0 = fp16 inputs (the reference), 1 = bf16 inputs (beyond the reference: same
- * algorithm, P still rounded to fp16).
+ * algorithm with P rounded to bf16, the type both operands of a bf16 matrix product share).
  */
 int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *sparseAToXidx,
                              const uint64_t *bitmap, int N, int d, int dtype, const uint16_t *Q,
@@ -382,12 +393,13 @@ int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *spar
             for (int i = 0; i < nb * 16; i++) {
               float ev = (S[i] == 0.0f) ? 0.0f : expf(S[i] - mnew);
               sum += ev;
-              P[i] = round_to_half(ev);
+              P[i] = dtype == 0 ? round_to_half(ev) : round_to_bf16(ev);
             }
             l = fmaf(alpha, l, sum);
             for (int c = 0; c < d; c++) O[c] *= alpha;
           } else {
-            for (int i = 0; i < nb * 16; i++) P[i] = round_to_half(S[i]);
+            for (int i = 0; i < nb * 16; i++)
+              P[i] = dtype == 0 ? round_to_half(S[i]) : round_to_bf16(S[i]);
           }
           for (int b = 0; b < nb; b++) {
             for (int j = 0; j < 16; j++) {

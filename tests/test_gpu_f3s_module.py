@@ -125,3 +125,35 @@ def test_module_argument_checks_on_device():
     # all-empty graph: every output row is zero
     out = F3S.f3s_1tb1rw(rwo, atox, bm, N, Q, Q, Q, 8, True, False)[1]
     assert float(out.abs().max()) == 0.0
+
+
+def test_multihead_entry_of_the_module(oracle_mod):
+    """F3S.f3s_multihead_scaleQK (bf16, [N, heads, d]) against the per-head loop the reference's
+    callers write with f3s_1tb1rw_scheduled_permuteV_scaleQK, and against the textbook oracle."""
+    print("case module_multihead", flush=True)
+    from fused3s_amd import F3S
+    N, heads, d = 1500, 8, 32
+    rowPtr, colIdx, _, _, _ = reference_style_inputs(N, d, density=0.03, seed=3)
+    res, _, _, _ = preprocess_like_the_reference(F3S, rowPtr, colIdx, N)
+    rwo, order, _, _, _, atox, bitmap, _ = res
+    g = torch.Generator().manual_seed(3)
+    Q, K, V = [(torch.randn((N, heads, d), generator=g) * d ** -0.5).to(torch.bfloat16).cuda()
+               for _ in range(3)]
+    scale = float(np.sqrt(d))
+    t, out, extra = F3S.f3s_multihead_scaleQK(rwo, order, atox, bitmap, N, Q, K, V, scale)
+    assert t.device.type == "cpu" and t.dim() == 0 and float(t) > 0
+    assert out.shape == (N, heads * d) and out.dtype == torch.float32 and extra.numel() == 0
+    for h in range(heads):
+        qh, kh, vh = (x[:, h].contiguous() for x in (Q, K, V))
+        _, single, _ = F3S.f3s_1tb1rw_scheduled_permuteV_scaleQK(rwo, order, atox, bitmap, N, qh,
+                                                                 kh, vh, scale, 8)
+        assert torch.equal(out[:, h * d:(h + 1) * d], single)
+        as_bits = lambda x: x.cpu().view(torch.int16).numpy().view(np.uint16)
+        txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, as_bits(qh), as_bits(kh),
+                                            as_bits(vh), scale, dtype=1)
+        assert np.abs(single.cpu().numpy() - txt).max() < MAX_ABS
+    with pytest.raises(RuntimeError, match="identical shapes"):
+        F3S.f3s_multihead_scaleQK(rwo, order, atox, bitmap, N, Q, K[:, :4], V, scale)
+    with pytest.raises(RuntimeError, match="float16 or all bfloat16"):
+        F3S.f3s_multihead_scaleQK(rwo, order, atox, bitmap, N, Q.float(), K.float(), V.float(),
+                                  scale)

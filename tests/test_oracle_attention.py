@@ -42,6 +42,39 @@ def test_half_conversions_match_numpy(oracle_mod):
     assert np.array_equal(got, want)
 
 
+def test_bf16_rounding_matches_torch(oracle_mod):
+    import torch
+    L = oracle_mod.lib()
+    rng = np.random.default_rng(1)
+    xs = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32),
+        (rng.standard_normal(2000) * 1e-20).astype(np.float32),
+        # ties and near-ties of the 8-bit mantissa, carry into the exponent
+        np.array([0.0, -0.0, 1.0, 1.00390625, 1.005859375, 1.0078125, 1.01171875, 1.99609375,
+                  1.998046875, 255.5, 3.0e38, 2.0 ** -126], np.float32)])
+    want = torch.from_numpy(xs).to(torch.bfloat16).to(torch.float32).numpy()
+    got = np.array([L.f3s_oracle_round_to_bf16(ctypes.c_float(float(x))) for x in xs], np.float32)
+    assert np.array_equal(got, want)
+
+
+def test_bf16_reference_emulation_matches_textbook(oracle_mod):
+    """bf16 inputs: same algorithm, P rounded to bf16; stays within max-abs 2e-2 of the fp64
+    textbook result and within a mean-relative error of 4e-3 (8-bit mantissa of P)."""
+    import torch
+    rng = np.random.default_rng(5)
+    N, d = 333, 64
+    rowPtr, colIdx = random_csr(rng, N, 20, hub=9, empty_frac=0.05)
+    g = torch.Generator().manual_seed(5)
+    Q, K, V = [torch.randn((N, d), generator=g).to(torch.bfloat16).view(torch.int16).numpy()
+               .view(np.uint16) for _ in range(3)]
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    ref = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                   N, Q, K, V, 8.0, dtype=1)
+    txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, 8.0, dtype=1)
+    assert np.abs(ref - txt).max() < MAX_ABS
+    assert 1e-5 < mean_rel(ref, txt) < 4e-3  # the bf16 rounding of P is visible, and bounded
+
+
 @pytest.mark.parametrize("seed,N,d,deg,dup,unsorted", [
     (0, 40, 32, 5, False, False), (1, 97, 64, 12, True, True), (2, 150, 128, 3, False, True)])
 def test_textbook_matches_dense_fp64(oracle_mod, seed, N, d, deg, dup, unsorted):
