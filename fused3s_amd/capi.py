@@ -15,7 +15,8 @@ _lib = None
 
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
            "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
-           "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads"]
+           "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads",
+           "f3s_attention_fwd_tcb8"]
 
 
 def lib():
@@ -45,6 +46,9 @@ def lib():
         L.f3s_attention_fwd_heads.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, ci, vp,
                                               vp, vp, ctypes.c_int64, ctypes.c_float, ci, vp,
                                               ctypes.c_int64, vp]
+        L.f3s_attention_fwd_tcb8.restype = ci
+        L.f3s_attention_fwd_tcb8.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, vp, vp, vp,
+                                             ci, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -193,3 +197,34 @@ def attention_heads(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, app
                                          int(bool(applySoftmax)), _ptr(out), out.stride(0),
                                          _stream()))
     return out
+
+
+def attention_tcb8(rwo, order, atox, bitmap, N, Q, K, V, applySoftmax=True, save_sddmm=False):
+    """f3s_attention_fwd_tcb8 on the current stream (16x8 TC blocks from preprocess(..., W=8)).
+    Returns out fp32[N, d], or (out, sddmm fp32[nTCB*128]) with save_sddmm."""
+    L = lib()
+    _dev(rwo, torch.int32, "rowWindowOffset")
+    _dev(atox, torch.int32, "sparseAToXidx")
+    _dev(bitmap, torch.uint64, "tcbBitMap")
+    for name, t in (("Q", Q), ("K", K), ("V", V)):
+        _dev(t, torch.float16, name)
+    if order is not None:
+        _dev(order, torch.int32, "windowOrder")
+        if order.numel() != rwo.numel() - 1:
+            raise RuntimeError("windowOrder must have one entry per row window")
+    d = Q.shape[1]
+    if Q.shape[0] < N or K.shape != Q.shape or V.shape != Q.shape:
+        raise RuntimeError("Q/K/V must be [N, d] with identical shapes")
+    if rwo.numel() != (N + 15) // 16 + 1:
+        raise RuntimeError("rowWindowOffset has %d entries, expected %d"
+                           % (rwo.numel(), (N + 15) // 16 + 1))
+    nT = atox.numel() // 8
+    if bitmap.numel() != 2 * nT:
+        raise RuntimeError("tcbBitMap must hold two words per 16x8 block")
+    out = torch.empty((N, d), dtype=torch.float32, device=Q.device)
+    sddmm = torch.empty(nT * 128, dtype=torch.float32, device=Q.device) if save_sddmm else None
+    with torch.cuda.device(Q.device):
+        _check(L.f3s_attention_fwd_tcb8(_ptr(rwo), _ptr(order), _ptr(atox), _ptr(bitmap), N, nT, d,
+                                        _ptr(Q), _ptr(K), _ptr(V), int(bool(applySoftmax)),
+                                        _ptr(out), _ptr(sddmm), _stream()))
+    return (out, sddmm) if save_sddmm else out

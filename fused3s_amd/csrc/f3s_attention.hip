@@ -113,14 +113,20 @@ __device__ __forceinline__ unsigned cu_key() {
 // out is [N, nHeads * D] with a row pitch of ldOut floats, and blockIdx.x = position * nHeads +
 // head, so that the workgroups of one window's heads are dispatched together and share the
 // window's column ids and bitmaps (and the neighbouring pieces of its K/V rows) in L2.
-template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS>
+// W8 = true: the structure comes from preprocessing with 8-column blocks (the reference's
+// 1tb1tcb path, src/F3S_kernel.cu:677-877). Column ids and bitmap words of two consecutive 16x8
+// blocks are laid out exactly like one 16x16 block, so the same pair pipeline runs over four
+// 16x8 blocks per step; rowWindowOffset then counts 16x8 blocks, a window may end in the middle
+// of a pair, and sddmm (if not null) receives the masked, unscaled scores, row-major 16x8 per
+// block (saveSddmmResult, src/F3S_kernel.cu:99-115).
+template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS, bool W8>
 __global__ __launch_bounds__(NWAVES * 64)
 __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
     int nRW, const ET* __restrict__ Q, const ET* __restrict__ K, const ET* __restrict__ V,
     float scaleLog2, float* __restrict__ out, unsigned long long* __restrict__ cuTimer,
-    int nHeads, int ldIn, int ldOut) {
+    int nHeads, int ldIn, int ldOut, float* __restrict__ sddmm) {
   typedef typename Vec<ET, 8>::type half8;
   constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
   unsigned long long tBegin = 0;
@@ -152,7 +158,8 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
 
   const int t0 = rowWindowOffset[w];
   const int t1 = rowWindowOffset[w + 1];
-  const int nPairs = (t1 - t0 + 1) >> 1;
+  constexpr int BPP = W8 ? 4 : 2;  // blocks of the structure per pipeline step
+  const int nPairs = (t1 - t0 + BPP - 1) / BPP;
 
   // B operand of the score product: this lane's query row, features 32i + 8g .. +7
   typedef int int4v __attribute__((ext_vector_type(4)));
@@ -182,17 +189,31 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   // the second block of the window's last pair may not exist: it aliases the first one
   // (loads stay in bounds) and its bits are cleared at use
   auto load_index = [&](int p) {
-    const int64_t tA = t0 + 2 * p;
-    const bool hasB = (tA + 1) < t1;
-    // lane -> dword index inside the pair's 32 ids / 16 bitmap dwords (second block folded onto
-    // the first when it does not exist)
-    const int idSlot = (lane & 31) & (hasB ? 31 : 15);
-    const int bmSlot = (lane & 15) & (hasB ? 15 : 7);
-    const int32_t* src = (lane < 32)
-                             ? sparseAToXidx + tA * 16 + idSlot
-                             : reinterpret_cast<const int32_t*>(bitmapBytes) + tA * 8 + bmSlot;
     PairIndex ix;
-    ix.meta = *src;
+    if constexpr (W8) {
+      // 8 ids and 4 bitmap dwords per block; blocks past the window's end fold onto the first
+      const int64_t tA = t0 + 4 * p;
+      const int nValid = (t1 - tA) < 4 ? (int)(t1 - tA) : 4;
+      int idSlot = lane & 31;
+      if (idSlot >= nValid * 8) idSlot &= 7;
+      int bmSlot = lane & 15;
+      if (bmSlot >= nValid * 4) bmSlot &= 3;
+      const int32_t* src = (lane < 32)
+                               ? sparseAToXidx + tA * 8 + idSlot
+                               : reinterpret_cast<const int32_t*>(bitmapBytes) + tA * 4 + bmSlot;
+      ix.meta = *src;
+    } else {
+      const int64_t tA = t0 + 2 * p;
+      const bool hasB = (tA + 1) < t1;
+      // lane -> dword index inside the pair's 32 ids / 16 bitmap dwords (second block folded
+      // onto the first when it does not exist)
+      const int idSlot = (lane & 31) & (hasB ? 31 : 15);
+      const int bmSlot = (lane & 15) & (hasB ? 15 : 7);
+      const int32_t* src = (lane < 32)
+                               ? sparseAToXidx + tA * 16 + idSlot
+                               : reinterpret_cast<const int32_t*>(bitmapBytes) + tA * 8 + bmSlot;
+      ix.meta = *src;
+    }
     return ix;
   };
   auto lane_read = [&](int v, int srcLane) { return __builtin_amdgcn_ds_bpermute(srcLane * 4, v); };
@@ -237,9 +258,13 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     return __builtin_bit_cast(half8, x);
   };
   auto compute = [&](const PairData<ET, D>& pd, int p) {
-    const bool hasB = (t0 + 2 * p + 1) < t1;
-    const unsigned bitsA = (pd.maskA >> maskShift) & 0xFu;
-    const unsigned bitsB = hasB ? ((pd.maskB >> maskShift) & 0xFu) : 0u;
+    // this lane's slots 4g..4g+3 of block A / B exist? (16x8 structure: they belong to block
+    // g/2 resp. 2 + g/2 of the step's four)
+    const int tFirst = t0 + BPP * p;
+    const bool validA = W8 ? (tFirst + (g >> 1)) < t1 : true;
+    const bool validB = W8 ? (tFirst + 2 + (g >> 1)) < t1 : (tFirst + 1) < t1;
+    const unsigned bitsA = validA ? ((pd.maskA >> maskShift) & 0xFu) : 0u;
+    const unsigned bitsB = validB ? ((pd.maskB >> maskShift) & 0xFu) : 0u;
     float4v sA = {0.f, 0.f, 0.f, 0.f}, sB = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < KS; i++) {
@@ -251,6 +276,14 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     for (int i = 0; i < 4; i++) {
       s[i] = ((bitsA >> (3 - i)) & 1u) ? sA[i] : 0.0f;
       s[4 + i] = ((bitsB >> (3 - i)) & 1u) ? sB[i] : 0.0f;
+    }
+    if constexpr (W8) {
+      if (sddmm) {
+        // lane (g, c): row c, columns 4(g&1)..+3 of block tFirst + g/2 (A) and + 2 (B)
+        float* dst = sddmm + ((size_t)(tFirst + (g >> 1)) * 16 + c) * 8 + 4 * (g & 1);
+        if (validA) *reinterpret_cast<float4*>(dst) = float4{s[0], s[1], s[2], s[3]};
+        if (validB) *reinterpret_cast<float4*>(dst + 256) = float4{s[4], s[5], s[6], s[7]};
+      }
     }
     half8 pf;
     if constexpr (SOFTMAX) {
@@ -399,18 +432,34 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
   const auto* v = static_cast<const ET*>(V);
   const dim3 block(NWAVES * 64);
   if (hl.nHeads > 0)
-    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, true>),
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, true, false>),
                        dim3((unsigned)nRW * (unsigned)hl.nHeads), block, 0, stream, rwo, order,
                        atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer, hl.nHeads, hl.ldIn,
-                       hl.ldOut);
+                       hl.ldOut, nullptr);
   else if (cuTimer)
-    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, true, false>), dim3(nRW), block, 0,
-                       stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer, 1,
-                       D, D);
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, true, false, false>), dim3(nRW),
+                       block, 0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out,
+                       cuTimer, 1, D, D, nullptr);
   else
-    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false>), dim3(nRW), block,
-                       0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer,
-                       1, D, D);
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false, false>), dim3(nRW),
+                       block, 0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out,
+                       cuTimer, 1, D, D, nullptr);
+  F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+template <int D, bool SOFTMAX>
+int launch_tcb8(const int32_t* rwo, const int32_t* order, const int32_t* atox,
+                const uint64_t* bitmap, int N, const void* Q, const void* K, const void* V,
+                float scaleLog2, float* out, float* sddmm, hipStream_t stream) {
+  constexpr int NWAVES = 4;
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  if (nRW == 0) return 0;
+  hipLaunchKernelGGL((f3s_fwd_kernel<_Float16, D, NWAVES, SOFTMAX, false, false, true>),
+                     dim3(nRW), dim3(NWAVES * 64), 0, stream, rwo, order, atox,
+                     reinterpret_cast<const uint8_t*>(bitmap), N, nRW,
+                     static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
+                     static_cast<const _Float16*>(V), scaleLog2, out, nullptr, 1, D, D, sddmm);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -474,6 +523,32 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                     : dispatch_d<__bf16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d,
                                          Q, K, V, scaleLog2, applySoftmax, out, cuTimer, single,
                                          stream);
+}
+
+int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                          const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                          const void* Q, const void* K, const void* V, int applySoftmax,
+                          float* out, float* sddmm, hipStream_t stream) {
+  if ((int64_t)N * d * 2 >= (int64_t)1 << 32)
+    return fail(-2, "f3s_attention_fwd_tcb8: K and V must each be smaller than 4 GiB");
+  // this path has no score scaling (src/F3S_kernel.cu:709-735)
+  const float scaleLog2 = applySoftmax ? kLog2e : 1.0f;
+#define F3S_DISPATCH(DD)                                                                      \
+  case DD:                                                                                    \
+    return applySoftmax ? launch_tcb8<DD, true>(rowWindowOffset, windowOrder, sparseAToXidx,  \
+                                                bitmap, N, Q, K, V, scaleLog2, out, sddmm,    \
+                                                stream)                                       \
+                        : launch_tcb8<DD, false>(rowWindowOffset, windowOrder, sparseAToXidx, \
+                                                 bitmap, N, Q, K, V, scaleLog2, out, sddmm,   \
+                                                 stream);
+  switch (d) {
+    F3S_DISPATCH(32)
+    F3S_DISPATCH(64)
+    F3S_DISPATCH(128)
+    default:
+      return fail(-2, "f3s_attention_fwd_tcb8: head dim %d unsupported (32, 64, 128)", d);
+  }
+#undef F3S_DISPATCH
 }
 
 int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,

@@ -119,4 +119,24 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
                                      out, ldOut, static_cast<hipStream_t>(stream));
 }
 
+int f3s_attention_fwd_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                           const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
+                           int64_t nTCB, int d, const void* Q, const void* K, const void* V,
+                           int applySoftmax, float* out, float* sddmmResult, void* stream) {
+  if (N < 0) return f3s::fail(-2, "f3s_attention_fwd_tcb8: negative N");
+  if (N == 0) return 0;
+  if (!rowWindowOffset || !Q || !K || !V || !out)
+    return f3s::fail(-1, "f3s_attention_fwd_tcb8: null pointer");
+  if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
+      f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 4) ||
+      f3s::misaligned(tcbBitMap, 8) || f3s::misaligned(sddmmResult, 16))
+    return f3s::fail(-1, "f3s_attention_fwd_tcb8: Q/K/V/out/sddmmResult need 16-byte alignment");
+  if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd_tcb8: negative nTCB");
+  if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
+    return f3s::fail(-1, "f3s_attention_fwd_tcb8: null TC-block arrays");
+  return f3s::launch_attention_tcb8(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, d,
+                                    Q, K, V, applySoftmax, out, sddmmResult,
+                                    static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

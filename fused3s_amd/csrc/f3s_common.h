@@ -34,6 +34,11 @@ int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* window
                            const void* V, int64_t ldIn, float scalingFactor, int applySoftmax,
                            float* out, int64_t ldOut, hipStream_t stream);
 
+int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                          const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                          const void* Q, const void* K, const void* V, int applySoftmax,
+                          float* out, float* sddmm, hipStream_t stream);
+
 // column-band schedule (f3s_attention_band.hip)
 size_t attention_workspace_bytes(int N, int d);
 int launch_attention_band(const int32_t* rowWindowOffset, const int32_t* windowOrder,

@@ -318,9 +318,9 @@ std::vector<torch::Tensor> f3s1tb1rwScheduledPermuteVScaleQK(
   return run_1tb1rw(rowWindowOffset, sparseAToXidx, tcbBitMap, nNodes, Q, K, V, nWarpPerBlock, L);
 }
 
-// F3S.f3s_1tb1tcb (src/F3S.cpp:272-296): the 16x8 split-feature kernel is not part of this
-// build yet; the entry exists so that callers fail with a clear error instead of an
-// AttributeError.
+// F3S.f3s_1tb1tcb (src/F3S.cpp:272-296; launcher src/F3S_kernel.cu:325-391): 16x8 TC blocks from
+// preprocess_gpu(..., blockSize_w = 8), natural window order, no score scaling; with
+// saveSddmmResult the third tensor holds the masked scores, 16x8 row-major per block.
 std::vector<torch::Tensor> f3s1tb1tcb(torch::Tensor rowWindowOffset, torch::Tensor sparseAToXidx,
                                       torch::Tensor tcbBitMap, int nNodes, torch::Tensor Q,
                                       torch::Tensor K, torch::Tensor V, bool applySoftmax,
@@ -331,10 +331,32 @@ std::vector<torch::Tensor> f3s1tb1tcb(torch::Tensor rowWindowOffset, torch::Tens
   F3S_CHECK_INPUT(rowWindowOffset);
   F3S_CHECK_INPUT(sparseAToXidx);
   F3S_CHECK_INPUT(tcbBitMap);
-  TORCH_CHECK(false,
-              "f3s_1tb1tcb (16x8 TC blocks) is not implemented in this build; use the 16x16 "
-              "entry points (f3s_1tb1rw*)");
-  return {};
+  TORCH_CHECK(Q.dim() == 2 && K.sizes() == Q.sizes() && V.sizes() == Q.sizes(),
+              "Q, K, V must be [N, d] with identical shapes");
+  TORCH_CHECK(Q.scalar_type() == torch::kHalf && K.scalar_type() == torch::kHalf &&
+                  V.scalar_type() == torch::kHalf,
+              "Q, K, V must be float16");
+  TORCH_CHECK(Q.size(0) >= nNodes, "Q, K, V need at least nNodes rows");
+  const int64_t d = Q.size(1);
+  const int64_t nRW = rowWindowOffset.numel() - 1;
+  TORCH_CHECK(nRW == ((int64_t)nNodes + 15) / 16,
+              "rowWindowOffset does not match nNodes (expected ceil(nNodes/16)+1 entries)");
+  const int64_t nTcb = sparseAToXidx.numel() / 8;
+  TORCH_CHECK(tcbBitMap.numel() == 2 * nTcb,
+              "tcbBitMap must hold two words per 16x8 block (preprocess_gpu with blockSize_w = 8)");
+  c10::DeviceGuard guard(Q.device());
+  auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(Q.device());
+  auto out = torch::empty({(int64_t)nNodes, d}, f32);
+  auto sddmmResult = torch::empty({saveSddmmResult ? nTcb * 128 : 0}, f32);
+  const float ms = timed_launch("f3s_attention_fwd_tcb8", [&](void* stream) {
+    return f3s_attention_fwd_tcb8(
+        rowWindowOffset.data_ptr<int>(), nullptr, sparseAToXidx.data_ptr<int>(),
+        reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()), nNodes, nTcb, (int)d,
+        Q.data_ptr(), K.data_ptr(), V.data_ptr(), applySoftmax ? 1 : 0, out.data_ptr<float>(),
+        saveSddmmResult ? sddmmResult.data_ptr<float>() : nullptr, stream);
+  });
+  auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));
+  return {time, out, sddmmResult};
 }
 
 }  // namespace

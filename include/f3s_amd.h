@@ -142,6 +142,27 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
                             const void* K, const void* V, int64_t ldIn, float scalingFactor,
                             int applySoftmax, float* out, int64_t ldOut, void* stream);
 
+/*
+ * Fused SDDMM -> softmax -> SpMM over 16x8 TC blocks: replaces f3sCuda1tb1tcb and
+ * f3sKernel1tb1tcb (src/F3S_kernel.cu:325-391, 677-877), the path behind F3S.f3s_1tb1tcb
+ * (src/F3S.cpp:272-296).
+ *
+ *   rowWindowOffset [nRW+1], sparseAToXidx [nTCB*8], tcbBitMap [nTCB*2]   from preprocessing
+ *                                  with H = 16, W = 8
+ *   windowOrder [nRW] or NULL      launch order (the reference launches in natural order)
+ *   Q, K, V [N*d]                  fp16, row-major, contiguous; d in {32, 64, 128}
+ *   applySoftmax                   0 = SDDMM -> SpMM only; scores are never scaled on this path
+ *   out [N*d] float                fully written
+ *   sddmmResult                    NULL, or nTCB*128 floats: the masked scores of every block,
+ *                                  row-major 16x8 (saveSddmmResult, src/F3S_kernel.cu:99-115);
+ *                                  fully written
+ * Asynchronous on `stream`.
+ */
+int f3s_attention_fwd_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                           const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
+                           int64_t nTCB, int d, const void* Q, const void* K, const void* V,
+                           int applySoftmax, float* out, float* sddmmResult, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

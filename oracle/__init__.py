@@ -48,6 +48,9 @@ def lib():
         L.f3s_oracle_attention_ref.restype = ci
         L.f3s_oracle_attention_ref.argtypes = [i32p, i32p, u64p, ci, ci, ci, u16p, u16p, u16p,
                                                ctypes.c_float, ci, ci, ci, ci, f32p]
+        L.f3s_oracle_attention_tcb8.restype = ci
+        L.f3s_oracle_attention_tcb8.argtypes = [i32p, i32p, u64p, ci, ci, u16p, u16p, u16p, ci,
+                                                f32p, f32p]
         L.f3s_oracle_attention_textbook.restype = ci
         L.f3s_oracle_attention_textbook.argtypes = [i32p, i32p, ci, ci, ci, u16p, u16p, u16p,
                                                     ctypes.c_float, ci, ci, ci, f32p]
@@ -132,6 +135,27 @@ def attention_ref(rwo, atox, bitmap, N, Q, K, V, scalingFactor=1.0, nWarpPerBloc
                                     _p(out, ctypes.c_float))
     assert rc == 0, rc
     return out
+
+
+def attention_tcb8(rwo, atox, bitmap, N, Q, K, V, applySoftmax=True, save_sddmm=False):
+    """Reference-emulating 1tb1tcb kernel (src/F3S_kernel.cu:677-877) on 16x8 TC blocks from
+    preprocess(..., W=8). Returns out, or (out, sddmm fp32[nTCB*128]) with save_sddmm."""
+    L = lib()
+    Qb, Kb, Vb = _bits(Q), _bits(K), _bits(V)
+    d = Qb.shape[1]
+    out = np.zeros((N, d), np.float32)
+    rwo = _i32(rwo)
+    nT = int(rwo[-1])
+    atox = _i32(atox) if len(atox) else np.zeros(1, np.int32)
+    bitmap = np.ascontiguousarray(bitmap, dtype=np.uint64) if len(bitmap) else np.zeros(1, np.uint64)
+    sddmm = np.zeros(max(nT, 1) * 128, np.float32) if save_sddmm else None
+    rc = L.f3s_oracle_attention_tcb8(_p(rwo, ctypes.c_int32), _p(atox, ctypes.c_int32),
+                                     _p(bitmap, ctypes.c_uint64), N, d, _p(Qb, ctypes.c_uint16),
+                                     _p(Kb, ctypes.c_uint16), _p(Vb, ctypes.c_uint16),
+                                     int(bool(applySoftmax)), _p(out, ctypes.c_float),
+                                     _p(sddmm, ctypes.c_float) if save_sddmm else None)
+    assert rc == 0, rc
+    return (out, sddmm[:nT * 128]) if save_sddmm else out
 
 
 def attention_textbook(rowPtr, colIdx, N, Q, K, V, scalingFactor=1.0, dtype=0, rows=None,

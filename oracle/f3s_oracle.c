@@ -427,6 +427,102 @@ int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *spar
 }
 
 /*
+ * Reference-emulating fused 3S over 16x8 TC blocks, the "1tb1tcb" kernel:
+ *   f3sKernel1tb1tcb                               src/F3S_kernel.cu:677-877
+ *   launcher (sddmmResult sizing, padded output)   src/F3S_kernel.cu:325-391
+ * Inputs come from preprocessing with blockSize_w = 8: sparseAToXidx has 8 column ids per block,
+ * tcbBitMap two words per block, word = row/8, bit 63 - ((row%8)*8 + col) (addPartialSums,
+ * src/F3S_kernel.cu:143-163). Per window the blocks are taken two at a time (:702-705; the
+ * second one is skipped when the window's count is odd, :703-705,716):
+ *   S = Q K^T in fp32, summed over the warps' feature slices, masked entries forced to 0, no
+ *   scaling (:709-735); sddmmResult[t*128 + row*8 + col] = S (saveSddmmResult, :99-115: its
+ *   "block row major" 8x8 sub-block order is plain row-major over the 16x8 block);
+ *   running max starts at 0 and takes part with the masked zeros (:688-690,762-766);
+ *   E = (S == 0) ? 0 : exp(S - m_new) (:768-772); l = l*exp(m_old - m_new) + sum(E) from the
+ *   un-rounded E (:774-782); O *= exp(m_old - m_new) (:784-787); P = fp16(E) (:793-798);
+ *   O += P V in fp32 (:830-853); out = (l != 0) ? O/l : O (:856-866).
+ * applySoftmax == 0: P = fp16(S), no max/sum/normalisation (:801-819).
+ * sddmm may be NULL.
+ */
+int f3s_oracle_attention_tcb8(const int32_t *rowWindowOffset, const int32_t *sparseAToXidx,
+                              const uint64_t *bitmap, int N, int d, const uint16_t *Q,
+                              const uint16_t *K, const uint16_t *V, int applySoftmax, float *out,
+                              float *sddmm) {
+  int nRW = (N + 15) / 16;
+  float *Qf = to_float(Q, (int64_t)N * d, 0);
+  float *Kf = to_float(K, (int64_t)N * d, 0);
+  float *Vf = to_float(V, (int64_t)N * d, 0);
+  if (!Qf || !Kf || !Vf) return -2;
+#pragma omp parallel
+  {
+    float S[16], P[16];
+    float *O = (float *)malloc(sizeof(float) * (size_t)d);
+#pragma omp for schedule(dynamic, 4)
+    for (int w = 0; w < nRW; w++) {
+      int64_t t0 = rowWindowOffset[w], t1 = rowWindowOffset[w + 1];
+      for (int rl = 0; rl < 16; rl++) {
+        int64_t r = (int64_t)w * 16 + rl;
+        int live = r < N; /* rows past N have an all-zero Q fragment (setQFrag, :165-183) */
+        const float *q = live ? Qf + r * d : NULL;
+        float m = 0.0f, l = 0.0f;
+        for (int c = 0; c < d; c++) O[c] = 0.0f;
+        for (int64_t tc = t0; tc < t1; tc += 2) {
+          int nb = (t1 - tc) < 2 ? 1 : 2;
+          float mnew = m;
+          for (int b = 0; b < nb; b++) {
+            for (int j = 0; j < 8; j++) {
+              float s = 0.0f;
+              int bit = (int)((bitmap[(tc + b) * 2 + rl / 8] >> (63 - ((rl % 8) * 8 + j))) & 1ULL);
+              if (bit && live) {
+                const float *k = Kf + (int64_t)sparseAToXidx[(tc + b) * 8 + j] * d;
+                double acc = 0.0;
+                for (int c = 0; c < d; c++) acc += (double)q[c] * (double)k[c];
+                s = (float)acc;
+              }
+              S[b * 8 + j] = s;
+              if (sddmm) sddmm[(tc + b) * 128 + rl * 8 + j] = s;
+              if (s > mnew) mnew = s;
+            }
+          }
+          if (applySoftmax) {
+            float alpha = expf(m - mnew);
+            m = mnew;
+            float sum = 0.0f;
+            for (int i = 0; i < nb * 8; i++) {
+              float ev = (S[i] == 0.0f) ? 0.0f : expf(S[i] - mnew);
+              sum += ev;
+              P[i] = round_to_half(ev);
+            }
+            l = fmaf(alpha, l, sum);
+            for (int c = 0; c < d; c++) O[c] *= alpha;
+          } else {
+            for (int i = 0; i < nb * 8; i++) P[i] = round_to_half(S[i]);
+          }
+          for (int b = 0; b < nb; b++) {
+            for (int j = 0; j < 8; j++) {
+              float p = P[b * 8 + j];
+              if (p == 0.0f) continue;
+              const float *v = Vf + (int64_t)sparseAToXidx[(tc + b) * 8 + j] * d;
+              for (int c = 0; c < d; c++) O[c] += p * v[c];
+            }
+          }
+        }
+        if (!live) continue;
+        float inv = 1.0f;
+        if (applySoftmax && l != 0.0f) inv = 1.0f / l;
+        float *o = out + r * d;
+        for (int c = 0; c < d; c++) o[c] = O[c] * inv;
+      }
+    }
+    free(O);
+  }
+  free(Qf);
+  free(Kf);
+  free(Vf);
+  return 0;
+}
+
+/*
  * Textbook masked-softmax attention straight from CSR, fp64 accumulation:
  *   out[i,:] = sum_{j in N(i)} softmax_j(Q_i.K_j / scalingFactor) V_j ,
  * N(i) = DISTINCT columns of CSR row i, empty row => 0.

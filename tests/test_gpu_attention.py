@@ -168,3 +168,41 @@ def test_column_band_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
                                       pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
     got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, band=True)
     assert np.abs(got_n - want_n).max() < 2e-2 * max(1.0, np.abs(want_n).max())
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("seed,N,deg,hub", [(0, 300, 2, 0), (1, 500, 6, 7), (2, 77, 40, 0),
+                                            (3, 16, 1, 0)])
+def test_16x8_blocks_match_the_1tb1tcb_oracle(oracle_mod, d, seed, N, deg, hub):
+    """f3s_attention_fwd_tcb8 on windows of 1, 2, 3, ... 16x8 blocks (every tail length of the
+    four-block pipeline step), in natural and heavy-first order, with and without the SDDMM tap."""
+    from fused3s_amd import capi
+    print("case tcb8 d=%d seed=%d N=%d" % (d, seed, N), flush=True)
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, hub=hub, empty_frac=0.1)
+    Q, K, V = feats(rng, N, d, std=0.6)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N, 16, 8)
+    counts = np.diff(pre["rowWindowOffset"])
+    print("blocks per window: min %d max %d" % (counts.min(), counts.max()), flush=True)
+    dev = "cuda"
+    rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
+    atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
+    bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
+    order = torch.as_tensor(pre["sortedRowWindows"].astype(np.int32)).to(dev)
+    Qd, Kd, Vd = (torch.as_tensor(x).to(dev) for x in (Q, K, V))
+    for softmax in (True, False):
+        want, want_s = oracle_mod.attention_tcb8(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                                 pre["tcbBitMap"], N, Q, K, V, softmax,
+                                                 save_sddmm=True)
+        got, got_s = capi.attention_tcb8(rwo, None, atox, bm, N, Qd, Kd, Vd, softmax,
+                                         save_sddmm=True)
+        got2 = capi.attention_tcb8(rwo, order, atox, bm, N, Qd, Kd, Vd, softmax)
+        torch.cuda.synchronize()
+        assert torch.equal(got, got2)
+        got, got_s = got.cpu().numpy(), got_s.cpu().numpy()
+        assert np.isfinite(got).all()
+        if softmax:
+            assert np.abs(got - want).max() < MAX_ABS
+        assert mean_rel(got, want) < MEAN_REL
+        assert np.array_equal(got_s == 0, want_s == 0)
+        assert np.abs(got_s - want_s).max() <= 1e-5 * max(1.0, np.abs(want_s).max())

@@ -120,8 +120,11 @@ def test_module_argument_checks_on_device():
     Qbad = torch.zeros(N, 48, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError, match="head dim"):
         F3S.f3s_1tb1rw(rwo, atox, bm, N, Qbad, Qbad, Qbad, 8, True, False)
-    with pytest.raises(RuntimeError, match="not implemented"):
-        F3S.f3s_1tb1tcb(rwo, atox, bm, N, Q, Q, Q, True, False)
+    with pytest.raises(RuntimeError, match="two words per 16x8 block"):
+        # 16 column ids are two 16x8 blocks, which need four bitmap words
+        F3S.f3s_1tb1tcb(rwo, atox, bm[:2].contiguous(), N, Q, Q, Q, True, False)
+    with pytest.raises(RuntimeError, match="float16"):
+        F3S.f3s_1tb1tcb(rwo, atox, bm, N, Q.float(), Q.float(), Q.float(), True, False)
     # all-empty graph: every output row is zero
     out = F3S.f3s_1tb1rw(rwo, atox, bm, N, Q, Q, Q, 8, True, False)[1]
     assert float(out.abs().max()) == 0.0
@@ -157,3 +160,43 @@ def test_multihead_entry_of_the_module(oracle_mod):
     with pytest.raises(RuntimeError, match="float16 or all bfloat16"):
         F3S.f3s_multihead_scaleQK(rwo, order, atox, bitmap, N, Q.float(), K.float(), V.float(),
                                   scale)
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_1tb1tcb_call_sequence(oracle_mod, d):
+    """F3S.f3s_1tb1tcb the way scripts/tests/test_f3s_accuracy.py:96-146 drives it:
+    preprocess_gpu with 16x8 blocks, softmax on / off, SDDMM tap checked block by block."""
+    print("case module_1tb1tcb d=%d" % d, flush=True)
+    from fused3s_amd import F3S
+    N = 1000
+    rowPtr, colIdx, Q, K, V = reference_style_inputs(N, d, density=0.05, seed=d)
+    want_pre = oracle_mod.preprocess(rowPtr, colIdx, N, 16, 8)
+    res, bp, e2c, e2r = preprocess_like_the_reference(F3S, rowPtr, colIdx, N, W=8)
+    rwo, order, rowid, tile, toff, atox, bitmap, nT = res
+    got_pre = dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
+                   tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox, blockCount=nT,
+                   tcbBitMap=bitmap.cpu().view(torch.int64).numpy().view(np.uint64),
+                   blockPartition=bp, edgeToColumn=e2c, edgeToRow=e2r)
+    got_pre = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in got_pre.items()}
+    compare_preprocess(got_pre, want_pre)
+    Qd, Kd, Vd = (torch.as_tensor(x).cuda() for x in (Q, K, V))
+    for softmax in (True, False):
+        want, want_s = oracle_mod.attention_tcb8(want_pre["rowWindowOffset"],
+                                                 want_pre["sparseAToXidx"], want_pre["tcbBitMap"],
+                                                 N, Q, K, V, softmax, save_sddmm=True)
+        t, out, sddmm = F3S.f3s_1tb1tcb(rwo, atox, bitmap, N, Qd, Kd, Vd, softmax, True)
+        assert t.device.type == "cpu" and float(t) > 0
+        assert out.shape == (N, d) and sddmm.shape == (nT * 128,)
+        got = out.cpu().numpy()
+        if softmax:
+            assert np.abs(got - want).max() < MAX_ABS
+            assert np.abs(got - want).mean() / np.abs(want).mean() < MEAN_REL
+        else:
+            # no normalisation: outputs are sums of fp16(S) * V with |S| ~ d/4; relative bar only
+            assert np.abs(got - want).mean() / np.abs(want).mean() < MEAN_REL
+        # scores: fp32 MFMA accumulation of exact fp16 products against a double-precision sum
+        got_s = sddmm.cpu().numpy()
+        assert np.array_equal(got_s == 0, want_s == 0)
+        assert np.abs(got_s - want_s).max() <= 1e-5 * max(1.0, np.abs(want_s).max())
+        t2, out2, empty = F3S.f3s_1tb1tcb(rwo, atox, bitmap, N, Qd, Kd, Vd, softmax, False)
+        assert empty.numel() == 0 and torch.equal(out2, out)

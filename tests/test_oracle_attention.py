@@ -191,3 +191,50 @@ def test_sddmm_spmm_without_softmax(oracle_mod):
     S = (Q.astype(np.float64) @ K.astype(np.float64).T) * A
     want = S.astype(np.float16).astype(np.float64) @ V.astype(np.float64)
     assert np.abs(got - want).max() < 5e-3 * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("seed,N,d,deg", [(0, 100, 32, 7), (1, 333, 64, 30), (2, 50, 128, 3)])
+def test_tcb8_oracle_pinned_by_the_16x16_one_and_by_dense_scores(oracle_mod, seed, N, d, deg):
+    """The 16x8 kernel walks the same ascending column list two blocks (16 columns) at a time, so
+    it must reproduce the 16x16 oracle run with one block per chunk (nWarpPerBlock=2) bit for bit;
+    its SDDMM tap must equal the dense Q K^T sampled at the edges, block by block."""
+    rng = np.random.default_rng(seed)
+    rowPtr, colIdx = random_csr(rng, N, deg, hub=5, empty_frac=0.1)
+    Q, K, V = feats(rng, N, d, std=0.5)
+    p16 = oracle_mod.preprocess(rowPtr, colIdx, N, 16, 16)
+    p8 = oracle_mod.preprocess(rowPtr, colIdx, N, 16, 8)
+    for softmax in (True, False):
+        want = oracle_mod.attention_ref(p16["rowWindowOffset"], p16["sparseAToXidx"],
+                                        p16["tcbBitMap"], N, Q, K, V, 1.0, nWarpPerBlock=2,
+                                        applySoftmax=softmax)
+        got, sddmm = oracle_mod.attention_tcb8(p8["rowWindowOffset"], p8["sparseAToXidx"],
+                                               p8["tcbBitMap"], N, Q, K, V, softmax,
+                                               save_sddmm=True)
+        assert np.array_equal(got, want)
+    txt = oracle_mod.attention_textbook(rowPtr, colIdx, N, Q, K, V, 1.0)
+    got = oracle_mod.attention_tcb8(p8["rowWindowOffset"], p8["sparseAToXidx"], p8["tcbBitMap"], N,
+                                    Q, K, V, True)
+    assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL
+    # SDDMM tap: block t of window w, row r, slot j  <->  A[16w + r, sparseAToXidx[8t + j]]
+    A = dense_from_csr(rowPtr, colIdx, N)
+    S = Q.astype(np.float64) @ K.astype(np.float64).T
+    rwo = p8["rowWindowOffset"]
+    nT = int(rwo[-1])
+    assert sddmm.shape == (nT * 128,)
+    blocks = sddmm.reshape(nT, 16, 8)
+    seen = 0
+    for w in range(len(rwo) - 1):
+        rows = range(16 * w, min(16 * w + 16, N))
+        n_cols = len(np.unique(np.concatenate([colIdx[rowPtr[r]:rowPtr[r + 1]] for r in rows])))
+        for t in range(rwo[w], rwo[w + 1]):
+            cols = p8["sparseAToXidx"][8 * t:8 * t + 8]
+            for j in range(8):
+                padding = (t - rwo[w]) * 8 + j >= n_cols  # zero-filled slot, carries no bit
+                for r in range(16):
+                    row = 16 * w + r
+                    if not padding and row < N and A[row, cols[j]] != 0:
+                        assert blocks[t, r, j] == np.float32(S[row, cols[j]])
+                        seen += 1
+                    else:
+                        assert blocks[t, r, j] == 0.0
+    assert seen == int((A != 0).sum())
