@@ -99,9 +99,6 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
     ap.add_argument("--cpu-budget", type=float, default=12.0)
-    ap.add_argument("--no-workspace", action="store_true",
-                    help="do not give the attention call its scratch buffer (forces the "
-                         "workgroup-per-window kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -163,7 +160,9 @@ def main():
 
     order = None if args.natural_order else pre["sortedRowWindows"]
     out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
-    workspace = None if args.no_workspace else capi.attention_workspace(N, d, dev)
+    # scratch of the experimental column-sliced schedule, only when it is asked for
+    workspace = (capi.attention_workspace(N, d, dev)
+                 if os.environ.get("F3S_SCHEDULE") == "sliced" else None)
 
     if heads == 1:
         def step():

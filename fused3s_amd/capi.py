@@ -113,7 +113,7 @@ def preprocess(rowPtr, colIdx, N, H=16, W=16):
 
 
 def attention_workspace(N, d, device):
-    """Scratch tensor for attention(..., workspace=...) (column-band schedule)."""
+    """Scratch tensor for attention(..., workspace=...) (experimental column-sliced schedule)."""
     nbytes = lib().f3s_attention_workspace_bytes(N, d)
     return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device)
 

@@ -501,21 +501,18 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   // the reference divides unmasked scores by scalingFactor (src/F3S_kernel.cu:1666-1667);
   // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
-  // Experimental column-band schedule (f3s_attention_band.hip), opt-in with
-  // F3S_SCHEDULE=band in the environment plus a workspace: every wave walks the column range
-  // band by band so that K/V rows could be shared through L2. Measured on the 233k-node
-  // benchmark graph it is slower than the default (6.5 ms against 2.06 ms): waves owning heavy
-  // windows fall bands behind the others, the L2 hit rate stays at 45 %, and one wave per window
-  // leaves the long windows unsplit. It is kept, tested for correctness, as the base for a
-  // balanced version; the default is the workgroup-per-window kernel below.
-  static const bool bandSchedule = [] {
+  // Experimental column-sliced schedule (f3s_attention_sliced.hip), opt-in with
+  // F3S_SCHEDULE=sliced in the environment plus a workspace: (window, column slice) units, each
+  // XCD working on one slice at a time so that its K/V rows stay in that XCD's L2, and a merge
+  // kernel. On the 233k-node benchmark graph it cuts the L2 misses from 118 M to 45 M per launch
+  // and runs in 1.99 ms against 2.06 ms; the default stays the workgroup-per-window kernel.
+  static const bool slicedSchedule = [] {
     const char* e = getenv("F3S_SCHEDULE");
-    return e && strcmp(e, "band") == 0;
+    return e && strcmp(e, "sliced") == 0;
   }();
-  const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
-  if (bandSchedule && dtype == 0 && workspace && !cuTimer && d <= 64 && nRW >= 2048 && nTcb >= 64 * nRW)
-    return launch_attention_band(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
-                                 V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
+  if (slicedSchedule && dtype == 0 && workspace && !cuTimer)
+    return launch_attention_sliced(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
+                                   V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
   const HeadLayout single = {0, d, d};
   return dtype == 0 ? dispatch_d<_Float16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N,
                                            d, Q, K, V, scaleLog2, applySoftmax, out, cuTimer,

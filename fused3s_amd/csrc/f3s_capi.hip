@@ -72,7 +72,7 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
 size_t f3s_attention_workspace_bytes(int N, int d) {
   if (N < 0) N = 0;
   if (d < 32) d = 32;
-  return f3s::attention_workspace_bytes(N, d);
+  return f3s::attention_sliced_workspace_bytes(N, d);
 }
 
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,

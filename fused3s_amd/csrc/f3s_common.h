@@ -39,13 +39,13 @@ int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowO
                           const void* Q, const void* K, const void* V, int applySoftmax,
                           float* out, float* sddmm, hipStream_t stream);
 
-// column-band schedule (f3s_attention_band.hip)
-size_t attention_workspace_bytes(int N, int d);
-int launch_attention_band(const int32_t* rowWindowOffset, const int32_t* windowOrder,
-                          const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
-                          const void* Q, const void* K, const void* V, float scaleLog2,
-                          int applySoftmax, float* out, void* workspace, size_t wsBytes,
-                          hipStream_t stream);
+// column-sliced schedule (f3s_attention_sliced.hip)
+size_t attention_sliced_workspace_bytes(int N, int d);
+int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                            const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
+                            const void* Q, const void* K, const void* V, float scaleLog2,
+                            int applySoftmax, float* out, void* workspace, size_t wsBytes,
+                            hipStream_t stream);
 
 // preprocessing (f3s_preprocess.hip)
 size_t preprocess_workspace_bytes(int N, int E);

@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
+#include <cstdlib>
 #include <fstream>
 #include <iomanip>
 #include <map>
@@ -203,8 +204,10 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
     timer = torch::zeros({3 * nRW}, f32.dtype(torch::kInt64));
     timerPtr = reinterpret_cast<unsigned long long*>(timer.data_ptr());
   }
-  // scratch of the opt-in column-band schedule (F3S_SCHEDULE=band); unused otherwise
-  const size_t wsBytes = f3s_attention_workspace_bytes(nNodes, (int)d);
+  // scratch of the opt-in column-sliced schedule (F3S_SCHEDULE=sliced); not allocated otherwise
+  const char* schedule = std::getenv("F3S_SCHEDULE");
+  const bool sliced = schedule && std::string(schedule) == "sliced";
+  const size_t wsBytes = sliced ? f3s_attention_workspace_bytes(nNodes, (int)d) : 0;
   auto workspace = torch::empty({(int64_t)std::max<size_t>(wsBytes, 4)}, f32.dtype(torch::kUInt8));
   const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
   const float ms = timed_launch("f3s_attention_fwd", [&](void* stream) {
@@ -213,7 +216,7 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
         sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
         nNodes, sparseAToXidx.numel() / 16, (int)d, dtype, Q.data_ptr(), K.data_ptr(),
         V.data_ptr(), L.scalingFactor, L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr,
-        workspace.data_ptr(), wsBytes, stream);
+        sliced ? workspace.data_ptr() : nullptr, wsBytes, stream);
   });
   if (L.timerFile) write_cu_time(timer, nRW, L.timerFile);
   auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));

@@ -106,11 +106,11 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *                                  (the Clocked variants, src/F3S_kernel.cu:1178-1368, 1803-1997)
  *   workspace, ws_bytes            NULL / 0, or device scratch of
  *                                  f3s_attention_workspace_bytes(N, d) bytes (4-byte aligned).
- *                                  Only the experimental column-band schedule uses it (selected
- *                                  with F3S_SCHEDULE=band in the environment, for graphs with
- *                                  >= 2048 windows and >= 64 TC blocks per window; results agree
- *                                  with the default schedule within the tolerance of the
- *                                  summation order).
+ *                                  Only the experimental column-sliced schedule uses it
+ *                                  (F3S_SCHEDULE=sliced in the environment, fp16, no cuTimer):
+ *                                  per (window, column slice) partial results that a second
+ *                                  kernel merges. Results agree with the default schedule
+ *                                  within the tolerance of the summation order.
  * Asynchronous on `stream`.
  */
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
@@ -121,7 +121,8 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
 
 /*
  * Bytes of device scratch f3s_attention_fwd can use for a graph of N nodes at head dimension d
- * (per-window block ranges of the column bands). The reference's launchers
+ * (slice boundaries per window plus one partial (m, l, O) per window and slice: about
+ * 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers
  * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);

@@ -20,14 +20,14 @@ def mean_rel(a, b):
     return float(np.abs(a - b).mean() / max(np.abs(b).mean(), 1e-30))
 
 
-def gpu_attention(pre, N, Q, K, V, scale, order=None, softmax=True, band=False):
+def gpu_attention(pre, N, Q, K, V, scale, order=None, softmax=True, sliced=False):
     from fused3s_amd import capi
     dev = "cuda"
     rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
     atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
     bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
     od = None if order is None else torch.as_tensor(np.asarray(order, np.int32)).to(dev)
-    ws = capi.attention_workspace(N, Q.shape[1], dev) if band else None
+    ws = capi.attention_workspace(N, Q.shape[1], dev) if sliced else None
     out = capi.attention(rwo, od, atox, bm, N, torch.as_tensor(Q).to(dev),
                          torch.as_tensor(K).to(dev), torch.as_tensor(V).to(dev), scale, softmax,
                          workspace=ws)
@@ -136,14 +136,14 @@ def test_end_to_end_hip_preprocess_then_attention(oracle_mod):
     assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL
 
 
-@pytest.mark.skipif(os.environ.get("F3S_SCHEDULE") != "band",
-                    reason="experimental column-band schedule: run with F3S_SCHEDULE=band")
+@pytest.mark.skipif(os.environ.get("F3S_SCHEDULE") != "sliced",
+                    reason="experimental column-sliced schedule: run with F3S_SCHEDULE=sliced")
 @pytest.mark.parametrize("d", [32, 64])
-def test_column_band_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
-    """A graph dense enough for the column-band schedule (>= 2048 windows, >= 64 TC blocks per
+def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
+    """The column-sliced schedule on a dense power-law graph (>= 2048 windows, >= 64 TC blocks per
     window): its result must match the reference-emulating oracle within the tolerance and the
     workgroup-per-window kernel closely, for both window orders and without softmax."""
-    print("case band d=%d" % d, flush=True)
+    print("case sliced d=%d" % d, flush=True)
     from fused3s_amd import synth
     rp, ci = synth.make_graph("cfg3_chunglu_233k", scale=0.145)   # N = 33 779: N % 16 != 0
     N = rp.numel() - 1
@@ -159,14 +159,14 @@ def test_column_band_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
                                     pre["tcbBitMap"], N, Q, K, V, scale)
     plain = gpu_attention(pre, N, Q, K, V, scale, pre["sortedRowWindows"])
     for order in (pre["sortedRowWindows"], None):
-        got = gpu_attention(pre, N, Q, K, V, scale, order, band=True)
+        got = gpu_attention(pre, N, Q, K, V, scale, order, sliced=True)
         assert np.isfinite(got).all()
         assert np.abs(got - want).max() < MAX_ABS
         assert mean_rel(got, want) < MEAN_REL
         assert np.abs(got - plain).max() < 2e-3
     want_n = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
                                       pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
-    got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, band=True)
+    got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, sliced=True)
     assert np.abs(got_n - want_n).max() < 2e-2 * max(1.0, np.abs(want_n).max())
 
 
