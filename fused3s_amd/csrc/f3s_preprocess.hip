@@ -188,8 +188,8 @@ __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
   if (lane == 0) blockPartition[w] = (nUniq + W - 1) / W;
 }
 
-template <int W>
-__global__ __launch_bounds__(kBlock) void window_rank_kernel(
+template <int W, int TB>
+__global__ __launch_bounds__(TB) void window_rank_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
     int nPasses, int sortMax, int32_t* __restrict__ blockPartition,
     int32_t* __restrict__ edgeToColumn,
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
   uint32_t* bits = smem;                 // range/32 words
   uint32_t* pref = smem + (range >> 5);  // range/128 group prefixes
   __shared__ int sRow[17];
-  __shared__ unsigned sWaveTot[kBlock / 64];
+  __shared__ unsigned sWaveTot[TB / 64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -217,10 +217,10 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
   unsigned uniqueBefore = 0;
   for (int pass = 0; pass < nPasses; pass++) {
     const int lo = pass * range;
-    for (int i = tid; i < nGroups; i += kBlock)
+    for (int i = tid; i < nGroups; i += TB)
       reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
-    for (int e = eS + tid; e < eE; e += kBlock) {
+    for (int e = eS + tid; e < eE; e += TB) {
       const int col = colIdx[e];
       if ((unsigned)col >= (unsigned)N) {
         atomicOr(&hdr->error, 1);
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
     }
     __syncthreads();
     unsigned carry = uniqueBefore;
-    for (int gb = 0; gb < nGroups; gb += kBlock) {
+    for (int gb = 0; gb < nGroups; gb += TB) {
       const int gi = gb + tid;
       unsigned cnt = 0;
       if (gi < nGroups) {
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
       __syncthreads();
       unsigned waveOff = 0, tileTot = 0;
 #pragma unroll
-      for (int v = 0; v < kBlock / 64; v++) {
+      for (int v = 0; v < TB / 64; v++) {
         const unsigned t = sWaveTot[v];
         if (v < wave) waveOff += t;
         tileTot += t;
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
       carry += tileTot;
       __syncthreads();
     }
-    for (int e = eS + tid; e < eE; e += kBlock) {
+    for (int e = eS + tid; e < eE; e += TB) {
       const int col = colIdx[e];
       const unsigned rel = (unsigned)(col - lo);
       if ((unsigned)col < (unsigned)N && rel < (unsigned)range) {
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_kernel(
     uniqueBefore = carry;
     __syncthreads();
   }
-  for (int e = eS + tid; e < eE; e += kBlock) edgeToRow[e] = r0 + row_of_edge(sRow, e);
+  for (int e = eS + tid; e < eE; e += TB) edgeToRow[e] = r0 + row_of_edge(sRow, e);
   if (tid == 0) blockPartition[w] = (int)((uniqueBefore + W - 1) / W);
 }
 
@@ -392,8 +392,8 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
 }
 
 // ------------------------------------------------------------------ phase 2
-template <int W>
-__global__ __launch_bounds__(kBlock) void window_fill_kernel(
+template <int W, int TB>
+__global__ __launch_bounds__(TB) void window_fill_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
     const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
     long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(kBlock) void window_fill_kernel(
   __shared__ unsigned sCnt[TC * 16];            // [block][row] counts, then running positions
   __shared__ unsigned long long sBm[TC * WPT];  // bitmaps of the chunk
   __shared__ int sRow[17];
-  __shared__ unsigned sWaveTot[kBlock / 64];
+  __shared__ unsigned sWaveTot[TB / 64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -424,10 +424,10 @@ __global__ __launch_bounds__(kBlock) void window_fill_kernel(
 
   for (int tc0 = 0; tc0 < nb; tc0 += TC) {
     const int nt = min(TC, nb - tc0);
-    for (int i = tid; i < nt * 16; i += kBlock) sCnt[i] = 0;
-    for (int i = tid; i < nt * WPT; i += kBlock) sBm[i] = 0ull;
+    for (int i = tid; i < nt * 16; i += TB) sCnt[i] = 0;
+    for (int i = tid; i < nt * WPT; i += TB) sBm[i] = 0ull;
     __syncthreads();
-    for (int e = eS + tid; e < eE; e += kBlock) {
+    for (int e = eS + tid; e < eE; e += TB) {
       const int ec = edgeToColumn[e];
       const int t = (ec >> LOGW) - tc0;
       if ((unsigned)t < (unsigned)nt) {
@@ -441,7 +441,7 @@ __global__ __launch_bounds__(kBlock) void window_fill_kernel(
       }
     }
     __syncthreads();
-    for (int tb = 0; tb < nt; tb += kBlock) {
+    for (int tb = 0; tb < nt; tb += TB) {
       const int t = tb + tid;
       unsigned nnz = 0;
       if (t < nt) {
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(kBlock) void window_fill_kernel(
       __syncthreads();
       unsigned waveOff = 0, tileTot = 0;
 #pragma unroll
-      for (int v = 0; v < kBlock / 64; v++) {
+      for (int v = 0; v < TB / 64; v++) {
         const unsigned x = sWaveTot[v];
         if (v < wave) waveOff += x;
         tileTot += x;
@@ -494,7 +494,7 @@ __global__ __launch_bounds__(kBlock) void window_fill_kernel(
     }
     // tile ids: each wave replays whole rows in CSR order, so positions inside a TC block
     // follow the edge order (src/utils.cu:213-223)
-    for (int r = wave; r < 16; r += kBlock / 64) {
+    for (int r = wave; r < 16; r += TB / 64) {
       const int rs = sRow[r], re = sRow[r + 1];
       for (int eb = rs; eb < re; eb += 64) {
         const int e = eb + lane;
@@ -571,14 +571,18 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
       hipLaunchKernelGGL(window_rank_small_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
                          rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr);
     F3S_HIP_CHECK(hipGetLastError());
-    if (W == 16)
-      hipLaunchKernelGGL(window_rank_kernel<16>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
-                         colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,
-                         edgeToRow, hdr);
-    else
-      hipLaunchKernelGGL(window_rank_kernel<8>, dim3(nRW), dim3(kBlock), lds, stream, rowPtr,
-                         colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,
-                         edgeToRow, hdr);
+    // eight waves per window when windows are long (more loads and LDS atomics in flight)
+#define F3S_RANK(WW, TBB)                                                                     \
+  hipLaunchKernelGGL((window_rank_kernel<WW, TBB>), dim3(nRW), dim3(TBB), lds, stream, rowPtr, \
+                     colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,       \
+                     edgeToRow, hdr)
+    const bool big = (int64_t)E >= (int64_t)nRW * 2048;
+    if (W == 16) {
+      if (big) F3S_RANK(16, 512); else F3S_RANK(16, 256);
+    } else {
+      if (big) F3S_RANK(8, 512); else F3S_RANK(8, 256);
+    }
+#undef F3S_RANK
     F3S_HIP_CHECK(hipGetLastError());
   }
   hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
@@ -607,14 +611,19 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
     return 0;
   }
   auto bm = reinterpret_cast<unsigned long long*>(bitmap);
-  if (W == 16)
-    hipLaunchKernelGGL(window_fill_kernel<16>, dim3(nRW), dim3(kBlock), 0, stream, rowPtr, colIdx,
-                       N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid,
-                       tcblocktileId, tcblockOffset, sparseAToXidx, bm);
-  else
-    hipLaunchKernelGGL(window_fill_kernel<8>, dim3(nRW), dim3(kBlock), 0, stream, rowPtr, colIdx,
-                       N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid,
-                       tcblocktileId, tcblockOffset, sparseAToXidx, bm);
+  // Windows with thousands of edges get 16 waves (one per row in the tile-id replay, 32 waves
+  // per CU to hide the latency of the LDS atomics and the ballot chains); short windows keep 4.
+#define F3S_FILL(WW, TBB)                                                                       \
+  hipLaunchKernelGGL((window_fill_kernel<WW, TBB>), dim3(nRW), dim3(TBB), 0, stream, rowPtr,   \
+                     colIdx, N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid, \
+                     tcblocktileId, tcblockOffset, sparseAToXidx, bm)
+  const bool big = (int64_t)E >= (int64_t)nRW * 2048;
+  if (W == 16) {
+    if (big) F3S_FILL(16, 512); else F3S_FILL(16, 256);
+  } else {
+    if (big) F3S_FILL(8, 512); else F3S_FILL(8, 256);
+  }
+#undef F3S_FILL
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
