@@ -427,17 +427,30 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
     for (int i = tid; i < nt * 16; i += TB) sCnt[i] = 0;
     for (int i = tid; i < nt * WPT; i += TB) sBm[i] = 0ull;
     __syncthreads();
-    for (int e = eS + tid; e < eE; e += TB) {
-      const int ec = edgeToColumn[e];
-      const int t = (ec >> LOGW) - tc0;
-      if ((unsigned)t < (unsigned)nt) {
-        const int r = row_of_edge(sRow, e);
-        const int cl = ec & (W - 1);
-        atomicAdd(&sCnt[t * 16 + r], 1u);
-        // 8x8 sub-blocks in column-major order, row-major and MSB-first inside
-        const int sub = (cl >> 3) * (W / 8) + (r >> 3);
-        atomicOr(&sBm[t * WPT + sub], 1ull << (63 - ((r & 7) * 8 + (cl & 7))));
-        sparseAToXidx[(int64_t)(base + tc0 + t) * W + cl] = colIdx[e];
+    // four edges per thread and step, loads first: the LDS atomics of one edge then overlap the
+    // memory latency of the next ones
+    for (int e0 = eS + tid; e0 < eE; e0 += 4 * TB) {
+      int ecs[4], cols[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int e = e0 + u * TB;
+        ecs[u] = (e < eE) ? edgeToColumn[e] : -1;
+        cols[u] = (e < eE) ? colIdx[e] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int e = e0 + u * TB;
+        const int ec = ecs[u];
+        const int t = (ec >> LOGW) - tc0;
+        if (ec >= 0 && (unsigned)t < (unsigned)nt) {
+          const int r = row_of_edge(sRow, e);
+          const int cl = ec & (W - 1);
+          atomicAdd(&sCnt[t * 16 + r], 1u);
+          // 8x8 sub-blocks in column-major order, row-major and MSB-first inside
+          const int sub = (cl >> 3) * (W / 8) + (r >> 3);
+          atomicOr(&sBm[t * WPT + sub], 1ull << (63 - ((r & 7) * 8 + (cl & 7))));
+          sparseAToXidx[(int64_t)(base + tc0 + t) * W + cl] = cols[u];
+        }
       }
     }
     __syncthreads();
@@ -496,10 +509,12 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
     // follow the edge order (src/utils.cu:213-223)
     for (int r = wave; r < 16; r += TB / 64) {
       const int rs = sRow[r], re = sRow[r + 1];
+      int ecNext = (rs + lane < re) ? edgeToColumn[rs + lane] : 0;
       for (int eb = rs; eb < re; eb += 64) {
         const int e = eb + lane;
         const bool valid = e < re;
-        const int ec = valid ? edgeToColumn[e] : 0;
+        const int ec = ecNext;
+        ecNext = (e + 64 < re) ? edgeToColumn[e + 64] : 0;  // next batch, in flight during this one
         const int t = (ec >> LOGW) - tc0;
         const bool inr = valid && (unsigned)t < (unsigned)nt;
         unsigned long long peers = __ballot(inr);
