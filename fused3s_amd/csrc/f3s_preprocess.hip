@@ -33,10 +33,14 @@ constexpr int kRangeMax = 393216;  // columns per bitset pass: 48 KiB of bits + 
 constexpr int kSortMax = 1024;     // windows up to this many edges are ranked by a per-wave LDS sort
 constexpr int kFillChunk = 512;    // TC blocks held in LDS at once by window_fill_kernel
 
-// workspace header (bytes 0..255): int64 nTCB, int32 error flag
+// workspace header (bytes 0..255): int64 nTCB, int32 error flag, and the queue of windows too
+// long for the wave-per-window kernel (filled by window_rank_small_kernel, drained by
+// window_rank_kernel)
 struct WsHeader {
   long long nTcb;
   int error;
+  int nBig;     // entries in the queue
+  int nextBig;  // next entry to hand out
 };
 constexpr size_t kWsHeaderBytes = 256;
 
@@ -75,7 +79,7 @@ template <int W>
 __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int nRW,
     int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
-    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr) {
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, int32_t* __restrict__ bigList) {
   constexpr int WAVES = kBlock / 64;
   __shared__ uint32_t sKeys[WAVES][kSortMax];
   __shared__ uint32_t sUniq[WAVES][kSortMax];
@@ -94,7 +98,10 @@ __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
     if (lane == 0) blockPartition[w] = 0;
     return;
   }
-  if (n > kSortMax) return;  // ranked by window_rank_kernel
+  if (n > kSortMax) {  // left to window_rank_kernel, through the queue if there is one
+    if (bigList && lane == 0) bigList[atomicAdd(&hdr->nBig, 1)] = w;
+    return;
+  }
   uint32_t* keys = sKeys[wave];
   uint32_t* uniq = sUniq[wave];
   int P = 64;
@@ -191,28 +198,37 @@ __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
 template <int W, int TB>
 __global__ __launch_bounds__(TB) void window_rank_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
-    int nPasses, int sortMax, int32_t* __restrict__ blockPartition,
+    int nPasses, int32_t* __restrict__ blockPartition,
     int32_t* __restrict__ edgeToColumn,
-    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr) {
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
+    const int32_t* __restrict__ bigList) {
   extern __shared__ __align__(16) uint32_t smem[];
   uint32_t* bits = smem;                 // range/32 words
   uint32_t* pref = smem + (range >> 5);  // range/128 group prefixes
   __shared__ int sRow[17];
   __shared__ unsigned sWaveTot[TB / 64];
+  __shared__ int sTake;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int w = blockIdx.x;
+  // Two ways to find work. With a queue (graphs of mostly short windows) the grid is a fixed
+  // number of workgroups that drain it: an empty queue ends the kernel at once instead of one
+  // workgroup per window holding this kernel's large LDS allocation. Without one (graphs of long
+  // windows, where the appends to the queue would cost more than they save) workgroup b takes
+  // window b.
+  const int nBig = bigList ? hdr->nBig : 1;
+  while (true) {
+  __syncthreads();  // the previous window's reads of sRow / sTake are done
+  if (tid == 0) sTake = bigList ? atomicAdd(&hdr->nextBig, 1) : 0;
+  __syncthreads();
+  if (sTake >= nBig) break;
+  const int w = bigList ? bigList[sTake] : (int)blockIdx.x;
   const int r0 = w * 16;
   if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
   __syncthreads();
   const int eS = sRow[0], eE = sRow[16];
-  if (eS == eE) {
-    if (tid == 0) blockPartition[w] = 0;
-    return;
-  }
-  if (eE - eS <= sortMax) return;  // ranked by window_rank_small_kernel
+  if (!bigList && eE - eS <= kSortMax) break;  // ranked by window_rank_small_kernel
   const int nGroups = range >> 7;
   unsigned uniqueBefore = 0;
   for (int pass = 0; pass < nPasses; pass++) {
@@ -268,6 +284,8 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
   }
   for (int e = eS + tid; e < eE; e += TB) edgeToRow[e] = r0 + row_of_edge(sRow, e);
   if (tid == 0) blockPartition[w] = (int)((uniqueBefore + W - 1) / W);
+  if (!bigList) break;
+  }
 }
 
 // ------------------------------------------------- scan + window ordering
@@ -542,6 +560,8 @@ __global__ void set_tail_kernel(int32_t* tcblockOffset, long long nTcb, int E) {
 __global__ void clear_header_kernel(WsHeader* hdr) {
   hdr->nTcb = 0;
   hdr->error = 0;
+  hdr->nBig = 0;
+  hdr->nextBig = 0;
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -579,19 +599,25 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
     const int nPasses = (N + range - 1) / range;
     const size_t lds = (size_t)(range / 32 + range / 128) * sizeof(uint32_t);
     const int smallGrid = (nRW + kBlock / 64 - 1) / (kBlock / 64);
+    const bool big = (int64_t)E >= (int64_t)nRW * 2048;  // long windows on average
+    int32_t* queue = big ? nullptr : valsTmp;
     if (W == 16)
       hipLaunchKernelGGL(window_rank_small_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
-                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr);
+                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
+                         queue);
     else
       hipLaunchKernelGGL(window_rank_small_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
-                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr);
+                         rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
+                         queue);
     F3S_HIP_CHECK(hipGetLastError());
     // eight waves per window when windows are long (more loads and LDS atomics in flight)
 #define F3S_RANK(WW, TBB)                                                                     \
-  hipLaunchKernelGGL((window_rank_kernel<WW, TBB>), dim3(nRW), dim3(TBB), lds, stream, rowPtr, \
-                     colIdx, N, range, nPasses, kSortMax, blockPartition, edgeToColumn,       \
-                     edgeToRow, hdr)
-    const bool big = (int64_t)E >= (int64_t)nRW * 2048;
+  hipLaunchKernelGGL((window_rank_kernel<WW, TBB>), dim3(rankGrid), dim3(TBB), lds, stream,   \
+                     rowPtr, colIdx, N, range, nPasses, blockPartition,                       \
+                     edgeToColumn, edgeToRow, hdr, queue)
+    // the queue lives in the buffer finalize_count_kernel later uses for its values and is
+    // drained by at most 8 workgroups per CU
+    const int rankGrid = big ? nRW : (nRW < 2048 ? nRW : 2048);
     if (W == 16) {
       if (big) F3S_RANK(16, 512); else F3S_RANK(16, 256);
     } else {
