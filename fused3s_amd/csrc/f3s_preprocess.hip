@@ -424,11 +424,13 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
   __shared__ unsigned long long sBm[TC * WPT];  // bitmaps of the chunk
   __shared__ int sRow[17];
   __shared__ unsigned sWaveTot[TB / 64];
+  __shared__ unsigned sUnsorted;  // bit r: row r's columns are not strictly ascending
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int w = blockIdx.x;
+  if (tid == 0) sUnsorted = 0u;
   if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
   const int base = rowWindowOffset[w];
   const int nb = rowWindowOffset[w + 1] - base;
@@ -454,6 +456,18 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
         const int e = e0 + u * TB;
         ecs[u] = (e < eE) ? edgeToColumn[e] : -1;
         cols[u] = (e < eE) ? colIdx[e] : 0;
+      }
+      if (tc0 == 0) {
+        // once per window: which rows are strictly ascending (every edge against its left
+        // neighbour in the same row)
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int e = e0 + u * TB;
+          if (e < eE && e > eS) {
+            const int r = row_of_edge(sRow, e);
+            if (e > sRow[r] && colIdx[e - 1] >= cols[u]) atomicOr(&sUnsorted, 1u << r);
+          }
+        }
       }
 #pragma unroll
       for (int u = 0; u < 4; u++) {
@@ -523,9 +537,30 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
       carry += tileTot;
       __syncthreads();
     }
-    // tile ids: each wave replays whole rows in CSR order, so positions inside a TC block
-    // follow the edge order (src/utils.cu:213-223)
+    // Tile ids sit in CSR edge order inside a TC block (src/utils.cu:213-223): position =
+    // start of (block, row) + number of earlier edges of that row in the block. In a strictly
+    // ascending row those are exactly the bits left of the edge's own bit in the block's bitmap
+    // row, so every edge finds its place on its own.
+    const unsigned unsorted = sUnsorted;
+    for (int e = eS + tid; e < eE; e += TB) {
+      const int ec = edgeToColumn[e];
+      const int t = (ec >> LOGW) - tc0;
+      if ((unsigned)t >= (unsigned)nt) continue;
+      const int r = row_of_edge(sRow, e);
+      if ((unsorted >> r) & 1u) continue;
+      const int cl = ec & (W - 1);
+      const int shift = 8 * (7 - (r & 7));
+      unsigned before = 0;
+      if (W == 16 && cl >= 8)
+        before = __popc((unsigned)(sBm[t * WPT + (r >> 3)] >> shift) & 0xFFu);
+      const unsigned own =
+          (unsigned)(sBm[t * WPT + (cl >> 3) * (W / 8) + (r >> 3)] >> shift) & 0xFFu;
+      before += __popc(own >> (8 - (cl & 7)));
+      tcblocktileId[sCnt[t * 16 + r] + before] = (uint8_t)(r * W + cl);
+    }
+    // rows with repeated or descending columns: a wave replays the whole row in order
     for (int r = wave; r < 16; r += TB / 64) {
+      if (!((unsorted >> r) & 1u)) continue;
       const int rs = sRow[r], re = sRow[r + 1];
       int ecNext = (rs + lane < re) ? edgeToColumn[rs + lane] : 0;
       for (int eb = rs; eb < re; eb += 64) {
