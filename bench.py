@@ -80,12 +80,15 @@ def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
 
 
 def measured_traffic(args):
-    """HBM-side bytes per launch of the attention kernel from rocprofv3 (FETCH_SIZE x 2.000 +
-    WRITE_SIZE x 1.000, factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md).
-    Counters cannot be read from inside this process, so the figure is the recorded one and is
-    only given for the workload it was measured on."""
+    """HBM-side bytes per attention call from rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
+    factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md). Counters cannot
+    be read from inside this process, so the figure is the recorded one and is only given for the
+    workload and schedule it was measured on."""
     if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
-        return 14_644_661 * 1024
+        if os.environ.get("F3S_SCHEDULE") == "sliced":
+            # slice_index + f3s_fwd_sliced + f3s_merge_slices
+            return (2 * (42_394 + 2_573_930 + 262_572) + 512 + 524_196 + 58_268) * 1024
+        return (2 * 7_350_110 + 58_241) * 1024
     return None
 
 
