@@ -79,13 +79,13 @@ def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
                       "(%d rows, %d edges), %.1f s wall" % (step, rows_done, edges, spent)}
 
 
-def measured_traffic(args):
+def measured_traffic(args, sliced):
     """HBM-side bytes per attention call from rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
     factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md). Counters cannot
     be read from inside this process, so the figure is the recorded one and is only given for the
     workload and schedule it was measured on."""
     if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
-        if os.environ.get("F3S_SCHEDULE") == "sliced":
+        if sliced:
             # slice_index + f3s_fwd_sliced + f3s_merge_slices
             return (2 * (42_394 + 2_573_930 + 262_572) + 512 + 524_196 + 58_268) * 1024
         return (2 * 7_350_110 + 58_241) * 1024
@@ -163,9 +163,10 @@ def main():
 
     order = None if args.natural_order else pre["sortedRowWindows"]
     out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
-    # scratch of the experimental column-sliced schedule, only when it is asked for
-    workspace = (capi.attention_workspace(N, d, dev)
-                 if os.environ.get("F3S_SCHEDULE") == "sliced" else None)
+    # scratch of the column-sliced schedule, which the library picks for graphs with long windows
+    workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype)
+    log("attention schedule: %s" % ("column-sliced (%.0f MB workspace)" % (workspace.numel() / 1e6)
+                                    if workspace is not None else "workgroup per window"))
 
     if heads == 1:
         def step():
@@ -200,6 +201,15 @@ def main():
     b_gather = N * D * 2.0 + nTCB * (2 * 16 * D * 2.0 + 96.0 * heads) + 4.0 * N * D
     achieved = f_mfma / t_avg / 1e12
 
+    # the bound that binds on paper: t_roof = max(F_mfma / P_mfma, B_min / BW_hbm)
+    traffic = measured_traffic(args, workspace is not None)
+    if f_mfma / (PEAK_MFMA_F16_TFLOPS * 1e12) >= b_min / (PEAK_HBM_GBPS * 1e9):
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": traffic}
+    else:
+        gbps = b_min / t_avg / 1e9
+        roofline = {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic}
     result = {
         "metric": "fused_3s_attention_effective_tflops_d%d_%s%s"
                   % (d, cfg["dtype"], "" if heads == 1 else "_%dheads" % heads),
@@ -221,9 +231,8 @@ def main():
         "hbm_min_gbps": b_min / t_med / 1e9, "hbm_min_frac": b_min / t_med / 1e9 / PEAK_HBM_GBPS,
         "gather_gbps": b_gather / t_med / 1e9,
         "preprocess_ms": pre_ms, "preprocess_gedges_per_s": E / pre_ms / 1e6,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS,
-                     "traffic": measured_traffic(args)},
+        "schedule": "column-sliced" if workspace is not None else "window",
+        "roofline": roofline,
     }
     log("kernel: median %.3f ms  mean %.3f ms  effective %.1f TFLOP/s  MFMA %.1f TFLOP/s (%.1f%%)"
         % (t_med * 1e3, t_avg * 1e3, f_eff / t_med / 1e12, achieved,

@@ -16,7 +16,7 @@ _lib = None
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
            "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
            "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads",
-           "f3s_attention_fwd_tcb8"]
+           "f3s_attention_fwd_tcb8", "f3s_attention_uses_workspace"]
 
 
 def lib():
@@ -46,6 +46,8 @@ def lib():
         L.f3s_attention_fwd_heads.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, ci, vp,
                                               vp, vp, ctypes.c_int64, ctypes.c_float, ci, vp,
                                               ctypes.c_int64, vp]
+        L.f3s_attention_uses_workspace.restype = ci
+        L.f3s_attention_uses_workspace.argtypes = [ci, ctypes.c_int64, ci, ci]
         L.f3s_attention_fwd_tcb8.restype = ci
         L.f3s_attention_fwd_tcb8.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, vp, vp, vp,
                                              ci, vp, vp, vp]
@@ -112,9 +114,14 @@ def preprocess(rowPtr, colIdx, N, H=16, W=16):
                 edgeToRow=edgeToRow)
 
 
-def attention_workspace(N, d, device):
-    """Scratch tensor for attention(..., workspace=...) (experimental column-sliced schedule)."""
-    nbytes = lib().f3s_attention_workspace_bytes(N, d)
+def attention_workspace(N, d, device, nTCB=None, dtype=torch.float16):
+    """Scratch tensor for attention(..., workspace=...) (column-sliced schedule). With nTCB given,
+    returns None when the library would not use it for this problem."""
+    L = lib()
+    if nTCB is not None and not L.f3s_attention_uses_workspace(
+            N, int(nTCB), d, 0 if dtype == torch.float16 else 1):
+        return None
+    nbytes = L.f3s_attention_workspace_bytes(N, d)
     return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device)
 
 

@@ -487,6 +487,26 @@ int dispatch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox,
 
 }  // namespace
 
+// The column-sliced schedule (f3s_attention_sliced.hip: (window, column slice) units, every XCD
+// on one slice at a time so that its K/V rows stay in that XCD's L2, plus a merge kernel) pays off
+// on graphs with long windows: on the 233k-node benchmark graph (475 TC blocks per window) it
+// takes 1.66 / 1.94 / 3.67 ms at d = 32 / 64 / 128 against 2.27 / 2.11 / 6.05 ms for the
+// workgroup-per-window kernel, with 6.5 GB instead of 15.1 GB of traffic beyond L2 at d = 64.
+// Short windows would be cut into units of one or two blocks; they keep the window kernel.
+// F3S_SCHEDULE=window / =sliced in the environment overrides the choice.
+int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype) {
+  static const int forced = [] {
+    const char* e = getenv("F3S_SCHEDULE");
+    if (e && strcmp(e, "sliced") == 0) return 1;
+    if (e && strcmp(e, "window") == 0) return -1;
+    return 0;
+  }();
+  if (dtype != 0 || (d != 32 && d != 64 && d != 128) || N <= 0) return 0;
+  if (forced) return forced > 0;
+  const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
+  return nRW >= 2048 && nTcb >= 64 * nRW;
+}
+
 int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                      const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int64_t nTcb,
                      int d, int dtype, const void* Q, const void* K, const void* V,
@@ -501,16 +521,7 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   // the reference divides unmasked scores by scalingFactor (src/F3S_kernel.cu:1666-1667);
   // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
-  // Experimental column-sliced schedule (f3s_attention_sliced.hip), opt-in with
-  // F3S_SCHEDULE=sliced in the environment plus a workspace: (window, column slice) units, each
-  // XCD working on one slice at a time so that its K/V rows stay in that XCD's L2, and a merge
-  // kernel. On the 233k-node benchmark graph it cuts the L2 misses from 118 M to 45 M per launch
-  // and runs in 1.99 ms against 2.06 ms; the default stays the workgroup-per-window kernel.
-  static const bool slicedSchedule = [] {
-    const char* e = getenv("F3S_SCHEDULE");
-    return e && strcmp(e, "sliced") == 0;
-  }();
-  if (slicedSchedule && dtype == 0 && workspace && !cuTimer)
+  if (workspace && !cuTimer && attention_uses_workspace(N, nTcb, d, dtype))
     return launch_attention_sliced(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
                                    V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
   const HeadLayout single = {0, d, d};

@@ -75,6 +75,10 @@ size_t f3s_attention_workspace_bytes(int N, int d) {
   return f3s::attention_sliced_workspace_bytes(N, d);
 }
 
+int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype) {
+  return f3s::attention_uses_workspace(N, nTCB, d, dtype);
+}
+
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                       const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int64_t nTCB,
                       int d, int dtype, const void* Q, const void* K, const void* V,

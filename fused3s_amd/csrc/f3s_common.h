@@ -39,6 +39,8 @@ int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowO
                           const void* Q, const void* K, const void* V, int applySoftmax,
                           float* out, float* sddmm, hipStream_t stream);
 
+int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype);
+
 // column-sliced schedule (f3s_attention_sliced.hip)
 size_t attention_sliced_workspace_bytes(int N, int d);
 int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,

@@ -204,12 +204,12 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
     timer = torch::zeros({3 * nRW}, f32.dtype(torch::kInt64));
     timerPtr = reinterpret_cast<unsigned long long*>(timer.data_ptr());
   }
-  // scratch of the opt-in column-sliced schedule (F3S_SCHEDULE=sliced); not allocated otherwise
-  const char* schedule = std::getenv("F3S_SCHEDULE");
-  const bool sliced = schedule && std::string(schedule) == "sliced";
+  const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
+  // scratch of the column-sliced schedule, allocated only for the graphs the library uses it on
+  const bool sliced = !L.timerFile && f3s_attention_uses_workspace(
+                                          nNodes, sparseAToXidx.numel() / 16, (int)d, dtype) != 0;
   const size_t wsBytes = sliced ? f3s_attention_workspace_bytes(nNodes, (int)d) : 0;
   auto workspace = torch::empty({(int64_t)std::max<size_t>(wsBytes, 4)}, f32.dtype(torch::kUInt8));
-  const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
   const float ms = timed_launch("f3s_attention_fwd", [&](void* stream) {
     return f3s_attention_fwd(
         rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,

@@ -106,11 +106,11 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *                                  (the Clocked variants, src/F3S_kernel.cu:1178-1368, 1803-1997)
  *   workspace, ws_bytes            NULL / 0, or device scratch of
  *                                  f3s_attention_workspace_bytes(N, d) bytes (4-byte aligned).
- *                                  Only the experimental column-sliced schedule uses it
- *                                  (F3S_SCHEDULE=sliced in the environment, fp16, no cuTimer):
- *                                  per (window, column slice) partial results that a second
- *                                  kernel merges. Results agree with the default schedule
- *                                  within the tolerance of the summation order.
+ *                                  With it, graphs for which f3s_attention_uses_workspace()
+ *                                  returns 1 are computed by the column-sliced schedule: per
+ *                                  (window, column slice) partial results that a second kernel
+ *                                  merges. Results agree with the default schedule within the
+ *                                  tolerance of the summation order. Ignored with cuTimer.
  * Asynchronous on `stream`.
  */
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
@@ -126,6 +126,13 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
  * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);
+
+/*
+ * 1 if f3s_attention_fwd would use a workspace for this problem (fp16, at least 2048 row windows
+ * with 64 or more TC blocks each on average), else 0: callers can skip the allocation.
+ * F3S_SCHEDULE=window or =sliced in the environment forces 0 or 1.
+ */
+int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype);
 
 /*
  * The same fused kernel over nHeads attention heads in one launch: Q, K, V are [N, nHeads, d]

@@ -136,8 +136,6 @@ def test_end_to_end_hip_preprocess_then_attention(oracle_mod):
     assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL
 
 
-@pytest.mark.skipif(os.environ.get("F3S_SCHEDULE") != "sliced",
-                    reason="experimental column-sliced schedule: run with F3S_SCHEDULE=sliced")
 @pytest.mark.parametrize("d", [32, 64])
 def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
     """The column-sliced schedule on a dense power-law graph (>= 2048 windows, >= 64 TC blocks per
@@ -155,6 +153,12 @@ def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
     pre = oracle_mod.preprocess(rowPtr, colIdx, N)
     nRW = (N + 15) // 16
     assert nRW >= 2048 and pre["blockCount"] >= 64 * nRW
+    from fused3s_amd import capi
+    if os.environ.get("F3S_SCHEDULE") != "window":
+        assert capi.lib().f3s_attention_uses_workspace(N, int(pre["blockCount"]), d, 0) == 1
+    assert capi.lib().f3s_attention_uses_workspace(300, 2000, d, 0) == (
+        1 if os.environ.get("F3S_SCHEDULE") == "sliced" else 0)  # too few windows
+    assert capi.lib().f3s_attention_uses_workspace(N, int(pre["blockCount"]), d, 1) == 0  # bf16
     want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
                                     pre["tcbBitMap"], N, Q, K, V, scale)
     plain = gpu_attention(pre, N, Q, K, V, scale, pre["sortedRowWindows"])
