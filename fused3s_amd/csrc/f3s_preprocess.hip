@@ -236,14 +236,22 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
     for (int i = tid; i < nGroups; i += TB)
       reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
-    for (int e = eS + tid; e < eE; e += TB) {
-      const int col = colIdx[e];
-      if ((unsigned)col >= (unsigned)N) {
-        atomicOr(&hdr->error, 1);
-        continue;
+    // four edges per thread and step, loads first
+    for (int e0 = eS + tid; e0 < eE; e0 += 4 * TB) {
+      int cols[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) cols[u] = (e0 + u * TB < eE) ? colIdx[e0 + u * TB] : lo;
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        if (e0 + u * TB >= eE) continue;
+        const int col = cols[u];
+        if ((unsigned)col >= (unsigned)N) {
+          atomicOr(&hdr->error, 1);
+          continue;
+        }
+        const unsigned rel = (unsigned)(col - lo);
+        if (rel < (unsigned)range) atomicOr(&bits[rel >> 5], 1u << (rel & 31));
       }
-      const unsigned rel = (unsigned)(col - lo);
-      if (rel < (unsigned)range) atomicOr(&bits[rel >> 5], 1u << (rel & 31));
     }
     __syncthreads();
     unsigned carry = uniqueBefore;
@@ -268,15 +276,29 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
       carry += tileTot;
       __syncthreads();
     }
-    for (int e = eS + tid; e < eE; e += TB) {
-      const int col = colIdx[e];
-      const unsigned rel = (unsigned)(col - lo);
-      if ((unsigned)col < (unsigned)N && rel < (unsigned)range) {
-        const unsigned wd = rel >> 5;
-        unsigned rank = pref[wd >> 2];
-        for (unsigned k = wd & ~3u; k < wd; k++) rank += __popc(bits[k]);
-        rank += __popc(bits[wd] & ((1u << (rel & 31)) - 1u));
-        edgeToColumn[e] = (int)rank;
+    for (int e0 = eS + tid; e0 < eE; e0 += 4 * TB) {
+      int cols[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) cols[u] = (e0 + u * TB < eE) ? colIdx[e0 + u * TB] : -1;
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int col = cols[u];
+        const unsigned rel = (unsigned)(col - lo);
+        if ((unsigned)col < (unsigned)N && rel < (unsigned)range) {
+          // rank = set bits below this one: group prefix, then the whole 128-bit group read at
+          // once and masked
+          const unsigned wd = rel >> 5;
+          const uint4 grp = reinterpret_cast<const uint4*>(bits)[wd >> 2];
+          const unsigned words[4] = {grp.x, grp.y, grp.z, grp.w};
+          unsigned rank = pref[wd >> 2];
+#pragma unroll
+          for (unsigned k = 0; k < 4; k++) {
+            const unsigned keep = k < (wd & 3u) ? 0xFFFFFFFFu
+                                  : (k == (wd & 3u) ? ((1u << (rel & 31)) - 1u) : 0u);
+            rank += __popc(words[k] & keep);
+          }
+          edgeToColumn[e0 + u * TB] = (int)rank;
+        }
       }
     }
     uniqueBefore = carry;
