@@ -89,10 +89,10 @@ struct PairIndex {
   int meta;
 };
 
-// Waves per SIMD the kernel is held to. Two, not more: with three or four waves per SIMD the
-// extra windows in flight per XCD spread the K/V rows being gathered over more of the column
-// range than the 4 MiB L2 covers, and the kernel gets slower (measured 2.0 ms at two waves,
-// 2.6 ms at three on the 233k-node benchmark graph).
+// Waves per SIMD the kernel is held to. Two at D >= 64: measured on the 233k-node benchmark
+// graph 3.17 ms at one wave, 2.04 ms at two, 2.62 ms at three. The kernel is bound by instruction
+// issue on the SIMDs with the vector L1 close behind, so a third wave has little to add, and the
+// extra windows in flight per XCD spread the gather over more columns than the L2 holds.
 constexpr int waves_per_simd(int d) { return d <= 32 ? 4 : 2; }
 
 // Constant-rate (100 MHz) timestamp shared by all CUs, and an id of the CU this wave runs on:
