@@ -126,7 +126,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     const int32_t* __restrict__ sparseAToXidx, const uint8_t* __restrict__ bitmapBytes, int N,
     int nRW, const ET* __restrict__ Q, const ET* __restrict__ K, const ET* __restrict__ V,
     float scaleLog2, float* __restrict__ out, unsigned long long* __restrict__ cuTimer,
-    int nHeads, int ldIn, int ldOut, float* __restrict__ sddmm) {
+    int nHeads, int ldIn, int ldOut, float* __restrict__ sddmm, int minBlocks) {
   typedef typename Vec<ET, 8>::type half8;
   constexpr int T = D / 16;   // output tiles == halfs read per lane per V row
   unsigned long long tBegin = 0;
@@ -158,6 +158,9 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
 
   const int t0 = rowWindowOffset[w];
   const int t1 = rowWindowOffset[w + 1];
+  // windows of at most minBlocks blocks belong to the wave-per-window kernel of the same call
+  // (f3s_fwd_unit_kernel); -1 when this kernel computes every window
+  if (t1 - t0 <= minBlocks) return;
   constexpr int BPP = W8 ? 4 : 2;  // blocks of the structure per pipeline step
   const int nPairs = (t1 - t0 + BPP - 1) / BPP;
 
@@ -414,9 +417,11 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
 }
 
 struct HeadLayout {
-  int nHeads;  // 0: contiguous [N, d] single head
-  int ldIn;    // row pitch of Q/K/V in elements
-  int ldOut;   // row pitch of out in floats
+  int nHeads;       // 0: contiguous [N, d] single head
+  int ldIn;         // row pitch of Q/K/V in elements
+  int ldOut;        // row pitch of out in floats
+  int minBlocks;    // this kernel skips windows of at most minBlocks blocks (-1: none)
+  int gridWindows;  // positions of the window order this launch covers (<= nRW)
 };
 
 template <typename ET, int D, bool SOFTMAX>
@@ -431,19 +436,21 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
   const auto* k = static_cast<const ET*>(K);
   const auto* v = static_cast<const ET*>(V);
   const dim3 block(NWAVES * 64);
+  const unsigned gw = (unsigned)(hl.gridWindows < nRW ? hl.gridWindows : nRW);
+  if (gw == 0) return 0;
   if (hl.nHeads > 0)
     hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, true, false>),
-                       dim3((unsigned)nRW * (unsigned)hl.nHeads), block, 0, stream, rwo, order,
-                       atox, bm, N, nRW, q, k, v, scaleLog2, out, cuTimer, hl.nHeads, hl.ldIn,
-                       hl.ldOut, nullptr);
+                       dim3(gw * (unsigned)hl.nHeads), block, 0, stream, rwo, order, atox, bm, N,
+                       nRW, q, k, v, scaleLog2, out, cuTimer, hl.nHeads, hl.ldIn, hl.ldOut,
+                       nullptr, hl.minBlocks);
   else if (cuTimer)
-    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, true, false, false>), dim3(nRW),
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, true, false, false>), dim3(gw),
                        block, 0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out,
-                       cuTimer, 1, D, D, nullptr);
+                       cuTimer, 1, D, D, nullptr, hl.minBlocks);
   else
-    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false, false>), dim3(nRW),
+    hipLaunchKernelGGL((f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false, false>), dim3(gw),
                        block, 0, stream, rwo, order, atox, bm, N, nRW, q, k, v, scaleLog2, out,
-                       cuTimer, 1, D, D, nullptr);
+                       cuTimer, 1, D, D, nullptr, hl.minBlocks);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -459,7 +466,7 @@ int launch_tcb8(const int32_t* rwo, const int32_t* order, const int32_t* atox,
                      dim3(nRW), dim3(NWAVES * 64), 0, stream, rwo, order, atox,
                      reinterpret_cast<const uint8_t*>(bitmap), N, nRW,
                      static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
-                     static_cast<const _Float16*>(V), scaleLog2, out, nullptr, 1, D, D, sddmm);
+                     static_cast<const _Float16*>(V), scaleLog2, out, nullptr, 1, D, D, sddmm, -1);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -486,6 +493,29 @@ int dispatch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox,
 }
 
 }  // namespace
+
+// Graphs of short windows (a few TC blocks each) leave most of a four-wave workgroup idle and
+// pay its LDS merge for nothing. With a window order such a call is split: windows of at most
+// kShortWindowBlocks blocks go to the wave-per-window kernel, the others, with a heavy-first order
+// a prefix of at most nTcb / kShortWindowBlocks positions, stay with f3s_fwd_kernel, which skips
+// the short ones. An order that is not heavy-first stays correct (a long window outside the
+// prefix is computed by one wave). The two kernels run one after the other, so the split only
+// pays when long windows are rare: it is taken below 16 blocks per window on average (measured:
+// 100k-node 8-head layer 0.164 -> 0.101 ms and 0.248 -> 0.176 ms; an R-MAT graph with 16.6 blocks
+// per window and windows of up to 731 would go from 0.107 to 0.129 ms and is left alone).
+// Without an order nothing is split. F3S_SHORT_WINDOWS=0 in the environment turns it off.
+constexpr int kShortWindowBlocks = 32;
+bool split_short_windows(const int32_t* windowOrder, int nRW, int64_t nTcb, HeadLayout* hl) {
+  static const bool off = [] {
+    const char* e = getenv("F3S_SHORT_WINDOWS");
+    return e && strcmp(e, "0") == 0;
+  }();
+  if (off || !windowOrder || nRW < 1024 || nTcb >= (int64_t)16 * nRW) return false;
+  hl->minBlocks = kShortWindowBlocks;
+  const int64_t longMax = nTcb / (kShortWindowBlocks + 1) + 1;
+  hl->gridWindows = (int)(longMax < nRW ? longMax : nRW);
+  return true;
+}
 
 // The column-sliced schedule (f3s_attention_sliced.hip: (window, column slice) units, every XCD
 // on one slice at a time so that its K/V rows stay in that XCD's L2, plus a merge kernel) pays off
@@ -524,7 +554,15 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   if (workspace && !cuTimer && attention_uses_workspace(N, nTcb, d, dtype))
     return launch_attention_sliced(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
                                    V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
-  const HeadLayout single = {0, d, d};
+  const int nRWi = (N + kWinRows - 1) / kWinRows;
+  HeadLayout single = {0, d, d, -1, nRWi};
+  if (!cuTimer && split_short_windows(windowOrder, nRWi, nTcb, &single)) {
+    const int rc = launch_attention_short_windows(rowWindowOffset, windowOrder, sparseAToXidx,
+                                                  bitmap, N, d, dtype, Q, K, V, scaleLog2,
+                                                  applySoftmax, out, 0, d, d, kShortWindowBlocks,
+                                                  single.gridWindows, stream);
+    if (rc != 0) return rc;
+  }
   return dtype == 0 ? dispatch_d<_Float16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N,
                                            d, Q, K, V, scaleLog2, applySoftmax, out, cuTimer,
                                            single, stream)
@@ -561,7 +599,7 @@ int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowO
 
 int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                            const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
-                           int nHeads, int d, int dtype, const void* Q, const void* K,
+                           int64_t nTcb, int nHeads, int d, int dtype, const void* Q, const void* K,
                            const void* V, int64_t ldIn, float scalingFactor, int applySoftmax,
                            float* out, int64_t ldOut, hipStream_t stream) {
   if (dtype != 0 && dtype != 1)
@@ -583,7 +621,14 @@ int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* window
   if (nRW * nHeads >= ((int64_t)1 << 31))
     return fail(-2, "f3s_attention_fwd_heads: too many (window, head) workgroups");
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
-  const HeadLayout hl = {nHeads, (int)ldIn, (int)ldOut};
+  HeadLayout hl = {nHeads, (int)ldIn, (int)ldOut, -1, (int)nRW};
+  if (split_short_windows(windowOrder, (int)nRW, nTcb, &hl)) {
+    const int rc = launch_attention_short_windows(rowWindowOffset, windowOrder, sparseAToXidx,
+                                                  bitmap, N, d, dtype, Q, K, V, scaleLog2,
+                                                  applySoftmax, out, nHeads, (int)ldIn, (int)ldOut,
+                                                  kShortWindowBlocks, hl.gridWindows, stream);
+    if (rc != 0) return rc;
+  }
   return dtype == 0 ? dispatch_d<_Float16>(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N,
                                            d, Q, K, V, scaleLog2, applySoftmax, out, nullptr, hl,
                                            stream)

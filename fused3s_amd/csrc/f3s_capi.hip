@@ -119,7 +119,7 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd_heads: null TC-block arrays");
   return f3s::launch_attention_heads(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N,
-                                     nHeads, d, dtype, Q, K, V, ldIn, scalingFactor, applySoftmax,
+                                     nTCB, nHeads, d, dtype, Q, K, V, ldIn, scalingFactor, applySoftmax,
                                      out, ldOut, static_cast<hipStream_t>(stream));
 }
 

@@ -30,7 +30,7 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
 
 int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                            const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
-                           int nHeads, int d, int dtype, const void* Q, const void* K,
+                           int64_t nTcb, int nHeads, int d, int dtype, const void* Q, const void* K,
                            const void* V, int64_t ldIn, float scalingFactor, int applySoftmax,
                            float* out, int64_t ldOut, hipStream_t stream);
 
@@ -48,6 +48,13 @@ int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windo
                             const void* Q, const void* K, const void* V, float scaleLog2,
                             int applySoftmax, float* out, void* workspace, size_t wsBytes,
                             hipStream_t stream);
+
+int launch_attention_short_windows(const int32_t* rowWindowOffset, const int32_t* windowOrder,
+                                   const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
+                                   int d, int dtype, const void* Q, const void* K, const void* V,
+                                   float scaleLog2, int applySoftmax, float* out, int nHeads,
+                                   int ldIn, int ldOut, int maxBlocks, int longPrefix,
+                                   hipStream_t stream);
 
 // preprocessing (f3s_preprocess.hip)
 size_t preprocess_workspace_bytes(int N, int E);
