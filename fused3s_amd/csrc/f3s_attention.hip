@@ -531,7 +531,7 @@ int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype) {
     if (e && strcmp(e, "window") == 0) return -1;
     return 0;
   }();
-  if (dtype != 0 || (d != 32 && d != 64 && d != 128) || N <= 0) return 0;
+  if ((dtype != 0 && dtype != 1) || (d != 32 && d != 64 && d != 128) || N <= 0) return 0;
   if (forced) return forced > 0;
   const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
   return nRW >= 2048 && nTcb >= 64 * nRW;
@@ -552,8 +552,9 @@ int launch_attention(const int32_t* rowWindowOffset, const int32_t* windowOrder,
   // exponentials are taken in base 2, so log2(e) is folded into the same multiplier
   const float scaleLog2 = applySoftmax ? kLog2e / scalingFactor : 1.0f;
   if (workspace && !cuTimer && attention_uses_workspace(N, nTcb, d, dtype))
-    return launch_attention_sliced(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, Q, K,
-                                   V, scaleLog2, applySoftmax, out, workspace, wsBytes, stream);
+    return launch_attention_sliced(rowWindowOffset, windowOrder, sparseAToXidx, bitmap, N, d, dtype,
+                                   Q, K, V, scaleLog2, applySoftmax, out, workspace, wsBytes,
+                                   stream);
   const int nRWi = (N + kWinRows - 1) / kWinRows;
   HeadLayout single = {0, d, d, -1, nRWi};
   if (!cuTimer && split_short_windows(windowOrder, nRWi, nTcb, &single)) {

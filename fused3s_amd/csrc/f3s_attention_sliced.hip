@@ -428,7 +428,7 @@ int choose_phases(int N, int d) {
   return P;
 }
 
-template <int D, bool SOFTMAX>
+template <typename ET, int D, bool SOFTMAX>
 int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* atox,
                     const uint64_t* bitmap, int N, const void* Q, const void* K, const void* V,
                     float scaleLog2, float* out, int32_t* sliceStart, float* partial, int P,
@@ -441,11 +441,11 @@ int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* ato
                      stream, rwo, atox, nRW, S, sliceWidth, sliceStart);
   F3S_HIP_CHECK(hipGetLastError());
   const int nGroups = (nRW + kUnitWaves - 1) / kUnitWaves;
-  hipLaunchKernelGGL((f3s_fwd_unit_kernel<_Float16, D, SOFTMAX, true, false>),
+  hipLaunchKernelGGL((f3s_fwd_unit_kernel<ET, D, SOFTMAX, true, false>),
                      dim3((unsigned)(P * nGroups * kXcds)), dim3(kUnitWaves * 64), 0, stream, order,
                      rwo, atox, reinterpret_cast<const uint8_t*>(bitmap), sliceStart, S, nGroups, N,
-                     nRW, static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
-                     static_cast<const _Float16*>(V), scaleLog2, partial, out, 1, D, D, 0, 0);
+                     nRW, static_cast<const ET*>(Q), static_cast<const ET*>(K),
+                     static_cast<const ET*>(V), scaleLog2, partial, out, 1, D, D, 0, 0);
   F3S_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL((f3s_merge_slices_kernel<D, SOFTMAX>), dim3((unsigned)((nRW + 3) / 4)),
                      dim3(256), 0, stream, sliceStart, S, N, nRW, partial, out);
@@ -466,9 +466,9 @@ size_t attention_sliced_workspace_bytes(int N, int d) {
 
 int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                             const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
-                            const void* Q, const void* K, const void* V, float scaleLog2,
-                            int applySoftmax, float* out, void* workspace, size_t wsBytes,
-                            hipStream_t stream) {
+                            int dtype, const void* Q, const void* K, const void* V,
+                            float scaleLog2, int applySoftmax, float* out, void* workspace,
+                            size_t wsBytes, hipStream_t stream) {
   if (wsBytes < attention_sliced_workspace_bytes(N, d))
     return fail(-2, "f3s_attention_fwd: workspace %zu B < required %zu B", wsBytes,
                 attention_sliced_workspace_bytes(N, d));
@@ -477,24 +477,31 @@ int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windo
   int32_t* sliceStart = static_cast<int32_t*>(workspace);
   float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                             align256(nRW * ((size_t)P * kXcds + 1) * 4));
-#define F3S_SLICED(DD)                                                                         \
+#define F3S_SLICED(ET, DD)                                                                     \
   case DD:                                                                                     \
-    return applySoftmax ? launch_sliced_d<DD, true>(rowWindowOffset, windowOrder,              \
-                                                    sparseAToXidx, bitmap, N, Q, K, V,         \
-                                                    scaleLog2, out, sliceStart, partial, P,    \
-                                                    stream)                                    \
-                        : launch_sliced_d<DD, false>(rowWindowOffset, windowOrder,             \
-                                                     sparseAToXidx, bitmap, N, Q, K, V,        \
-                                                     scaleLog2, out, sliceStart, partial, P,   \
-                                                     stream);
-  switch (d) {
-    F3S_SLICED(32)
-    F3S_SLICED(64)
-    F3S_SLICED(128)
-    default:
-      return fail(-2, "f3s_attention_fwd: head dim %d unsupported (32, 64, 128)", d);
+    return applySoftmax ? launch_sliced_d<ET, DD, true>(rowWindowOffset, windowOrder,          \
+                                                        sparseAToXidx, bitmap, N, Q, K, V,     \
+                                                        scaleLog2, out, sliceStart, partial,   \
+                                                        P, stream)                             \
+                        : launch_sliced_d<ET, DD, false>(rowWindowOffset, windowOrder,         \
+                                                         sparseAToXidx, bitmap, N, Q, K, V,    \
+                                                         scaleLog2, out, sliceStart, partial,  \
+                                                         P, stream);
+  if (dtype == 0) {
+    switch (d) {
+      F3S_SLICED(_Float16, 32)
+      F3S_SLICED(_Float16, 64)
+      F3S_SLICED(_Float16, 128)
+    }
+  } else {
+    switch (d) {
+      F3S_SLICED(__bf16, 32)
+      F3S_SLICED(__bf16, 64)
+      F3S_SLICED(__bf16, 128)
+    }
   }
 #undef F3S_SLICED
+  return fail(-2, "f3s_attention_fwd: head dim %d unsupported (32, 64, 128)", d);
 }
 
 namespace {

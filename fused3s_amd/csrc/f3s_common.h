@@ -45,9 +45,9 @@ int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype);
 size_t attention_sliced_workspace_bytes(int N, int d);
 int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                             const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
-                            const void* Q, const void* K, const void* V, float scaleLog2,
-                            int applySoftmax, float* out, void* workspace, size_t wsBytes,
-                            hipStream_t stream);
+                            int dtype, const void* Q, const void* K, const void* V,
+                            float scaleLog2, int applySoftmax, float* out, void* workspace,
+                            size_t wsBytes, hipStream_t stream);
 
 int launch_attention_short_windows(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                                    const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,

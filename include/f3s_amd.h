@@ -128,8 +128,8 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
 size_t f3s_attention_workspace_bytes(int N, int d);
 
 /*
- * 1 if f3s_attention_fwd would use a workspace for this problem (fp16, at least 2048 row windows
- * with 64 or more TC blocks each on average), else 0: callers can skip the allocation.
+ * 1 if f3s_attention_fwd would use a workspace for this problem (at least 2048 row windows with
+ * 64 or more TC blocks each on average), else 0: callers can skip the allocation.
  * F3S_SCHEDULE=window or =sliced in the environment forces 0 or 1.
  */
 int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype);

@@ -158,7 +158,7 @@ def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
         assert capi.lib().f3s_attention_uses_workspace(N, int(pre["blockCount"]), d, 0) == 1
     assert capi.lib().f3s_attention_uses_workspace(300, 2000, d, 0) == (
         1 if os.environ.get("F3S_SCHEDULE") == "sliced" else 0)  # too few windows
-    assert capi.lib().f3s_attention_uses_workspace(N, int(pre["blockCount"]), d, 1) == 0  # bf16
+    assert capi.lib().f3s_attention_uses_workspace(N, int(pre["blockCount"]), 48, 0) == 0  # bad d
     want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
                                     pre["tcbBitMap"], N, Q, K, V, scale)
     plain = gpu_attention(pre, N, Q, K, V, scale, pre["sortedRowWindows"])
@@ -172,6 +172,23 @@ def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
                                       pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
     got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, sliced=True)
     assert np.abs(got_n - want_n).max() < 2e-2 * max(1.0, np.abs(want_n).max())
+    # bf16 inputs through the same schedule (P rounded to bf16: mean-relative bar 4e-3)
+    as_bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
+    Qb, Kb, Vb = (torch.as_tensor(x.astype(np.float32)).to(torch.bfloat16) for x in (Q, K, V))
+    want_b = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                      pre["tcbBitMap"], N, as_bits(Qb), as_bits(Kb), as_bits(Vb),
+                                      scale, dtype=1)
+    dev = "cuda"
+    rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
+    atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
+    bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
+    od = torch.as_tensor(pre["sortedRowWindows"].astype(np.int32)).to(dev)
+    ws = capi.attention_workspace(N, d, dev, nTCB=int(pre["blockCount"]), dtype=torch.bfloat16)
+    assert ws is not None or os.environ.get("F3S_SCHEDULE") == "window"
+    got_b = capi.attention(rwo, od, atox, bm, N, Qb.to(dev), Kb.to(dev), Vb.to(dev), scale,
+                           workspace=ws).cpu().numpy()
+    assert np.abs(got_b - want_b).max() < MAX_ABS
+    assert mean_rel(got_b, want_b) < 4e-3
 
 
 @pytest.mark.parametrize("d", [32, 64, 128])
