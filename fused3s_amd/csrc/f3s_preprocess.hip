@@ -317,49 +317,63 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     const int32_t* __restrict__ blockPartition, int nRW, int32_t* __restrict__ rowWindowOffset,
     int32_t* __restrict__ sortedRowWindows, int32_t* __restrict__ keysA,
     int32_t* __restrict__ keysB, int32_t* __restrict__ valsTmp, WsHeader* __restrict__ hdr) {
+  // One workgroup; every wave owns a contiguous chunk of the windows and walks it on its own
+  // (wave-level scans and ballots only), so a pass over the array costs a handful of block
+  // barriers instead of several per 1024 elements.
   constexpr int NW = kFinBlock / 64;
-  __shared__ unsigned sWave[NW];
-  __shared__ int sMax;
-  __shared__ unsigned sBinBase[16];
-  __shared__ unsigned sCnt[NW][16];
-  __shared__ unsigned sOff[NW][16];
-  __shared__ unsigned sTileTot[16];
+  __shared__ unsigned sWaveSum[NW];
+  __shared__ int sWaveMax[NW];
+  __shared__ unsigned sCnt[NW][16];   // per wave: elements per digit, then its running position
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int chunk = (((nRW + NW - 1) / NW) + 63) & ~63;
+  const int cBegin = min(wave * chunk, nRW);
+  const int cEnd = min(cBegin + chunk, nRW);
 
-  // inclusive scan of the block counts into rowWindowOffset[1..], and their maximum
-  if (tid == 0) sMax = 0;
-  __syncthreads();
-  unsigned carry = 0;
-  int localMax = 0;
-  for (int base = 0; base < nRW; base += kFinBlock) {
-    const int i = base + tid;
-    const unsigned v = (i < nRW) ? (unsigned)blockPartition[i] : 0u;
-    localMax = max(localMax, (int)v);
-    const unsigned incl = wave_inclusive_scan(v, lane);
-    if (lane == 63) sWave[wave] = incl;
-    __syncthreads();
-    unsigned waveOff = 0, tot = 0;
-#pragma unroll
-    for (int k = 0; k < NW; k++) {
-      const unsigned t = sWave[k];
-      if (k < wave) waveOff += t;
-      tot += t;
+  // ---- inclusive scan of the block counts into rowWindowOffset[1..], and their maximum
+  {
+    unsigned sum = 0;
+    int mx = 0;
+    for (int i = cBegin + lane; i < cEnd; i += 64) {
+      const int v = blockPartition[i];
+      sum += (unsigned)v;
+      mx = max(mx, v);
     }
-    if (i < nRW) rowWindowOffset[i + 1] = (int)(carry + waveOff + incl);
-    carry += tot;
-    __syncthreads();
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      sum += __shfl_xor(sum, off);
+      mx = max(mx, __shfl_xor(mx, off));
+    }
+    if (lane == 0) {
+      sWaveSum[wave] = sum;
+      sWaveMax[wave] = mx;
+    }
   }
-  atomicMax(&sMax, localMax);
+  __syncthreads();
+  unsigned carry = 0, total = 0;
+  int maxC = 0;
+#pragma unroll
+  for (int k = 0; k < NW; k++) {
+    const unsigned t = sWaveSum[k];
+    if (k < wave) carry += t;
+    total += t;
+    maxC = max(maxC, sWaveMax[k]);
+  }
+  for (int base = cBegin; base < cEnd; base += 64) {
+    const int i = base + lane;
+    const unsigned v = (i < cEnd) ? (unsigned)blockPartition[i] : 0u;
+    const unsigned incl = wave_inclusive_scan(v, lane);
+    if (i < cEnd) rowWindowOffset[i + 1] = (int)(carry + incl);
+    carry += __shfl(incl, 63);
+  }
   if (tid == 0) {
     rowWindowOffset[0] = 0;
-    hdr->nTcb = (long long)carry;
+    hdr->nTcb = (long long)total;
   }
-  __syncthreads();
-  const int maxC = sMax;
 
-  // stable sort by descending count == stable ascending LSD radix sort of (maxC - count)
+  // ---- stable sort by descending count == stable ascending LSD radix sort of (maxC - count),
+  // four bits per pass
   int nBits = 0;
   while ((maxC >> nBits) != 0) nBits++;
   const int nPass = (nBits + 3) / 4;
@@ -375,58 +389,63 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     int32_t* vDst = toOut ? sortedRowWindows : valsTmp;
     const int32_t* kSrc = toOut ? keysB : keysA;
     const int32_t* vSrc = toOut ? valsTmp : sortedRowWindows;
-    if (tid < 16) sBinBase[tid] = 0;
-    __syncthreads();
-    for (int i = tid; i < nRW; i += kFinBlock) {
-      const int key = (pass == 0) ? (maxC - blockPartition[i]) : kSrc[i];
-      atomicAdd(&sBinBase[(key >> shift) & 15], 1u);
-    }
-    __syncthreads();
-    if (tid == 0) {
-      unsigned run = 0;
-      for (int dgt = 0; dgt < 16; dgt++) {
-        const unsigned c = sBinBase[dgt];
-        sBinBase[dgt] = run;
-        run += c;
-      }
-    }
-    __syncthreads();
-    for (int base = 0; base < nRW; base += kFinBlock) {
-      const int i = base + tid;
-      const bool valid = i < nRW;
-      int key = 0, val = 0;
-      if (valid) {
-        key = (pass == 0) ? (maxC - blockPartition[i]) : kSrc[i];
-        val = (pass == 0) ? i : vSrc[i];
-      }
-      const int dgt = (key >> shift) & 15;
-      if (tid < NW * 16) (&sCnt[0][0])[tid] = 0;
-      __syncthreads();
+    __syncthreads();  // the previous pass's writes are visible, its use of sCnt is over
+    if (lane < 16) sCnt[wave][lane] = 0;
+    // peers = lanes of this 64-element group with the same digit (four ballots)
+    auto digit_peers = [&](bool valid, int dgt) {
       unsigned long long peers = __ballot(valid);
 #pragma unroll
       for (int b = 0; b < 4; b++) {
         const unsigned long long bal = __ballot((dgt >> b) & 1);
         peers &= ((dgt >> b) & 1) ? bal : ~bal;
       }
-      const unsigned rank = __popcll(peers & ltMask);
-      if (valid && rank == 0) sCnt[wave][dgt] = __popcll(peers);
-      __syncthreads();
-      if (tid < NW * 16) {
-        const int d2 = tid & 15, v2 = tid >> 4;
-        unsigned off = 0;
-        for (int k = 0; k < v2; k++) off += sCnt[k][d2];
-        sOff[v2][d2] = off;
-        if (v2 == NW - 1) sTileTot[d2] = off + sCnt[v2][d2];
-      }
-      __syncthreads();
+      return peers;
+    };
+    auto load_key = [&](int i) {
+      return (i < cEnd) ? ((pass == 0) ? (maxC - blockPartition[i]) : kSrc[i]) : 0;
+    };
+    auto load_val = [&](int i) { return (i < cEnd) ? ((pass == 0) ? i : vSrc[i]) : 0; };
+    // histogram of the wave's chunk (the next group's keys are in flight during this one's)
+    int keyNext = load_key(cBegin + lane);
+    for (int base = cBegin; base < cEnd; base += 64) {
+      const int i = base + lane;
+      const bool valid = i < cEnd;
+      const int key = keyNext;
+      keyNext = load_key(i + 64);
+      const int dgt = (key >> shift) & 15;
+      const unsigned long long peers = digit_peers(valid, dgt);
+      if (valid && (peers & ltMask) == 0ull) sCnt[wave][dgt] += __popcll(peers);
+    }
+    __syncthreads();
+    // start of (digit, wave): all smaller digits, then the same digit in earlier waves
+    unsigned start = 0;
+    if (lane < 16) {
+      for (int d2 = 0; d2 < 16; d2++)
+        for (int k = 0; k < NW; k++) {
+          const unsigned cnt = sCnt[k][d2];
+          if (d2 < lane || (d2 == lane && k < wave)) start += cnt;
+        }
+    }
+    __syncthreads();
+    if (lane < 16) sCnt[wave][lane] = start;
+    // scatter, in order
+    keyNext = load_key(cBegin + lane);
+    int valNext = load_val(cBegin + lane);
+    for (int base = cBegin; base < cEnd; base += 64) {
+      const int i = base + lane;
+      const bool valid = i < cEnd;
+      const int key = keyNext, val = valNext;
+      keyNext = load_key(i + 64);
+      valNext = load_val(i + 64);
+      const int dgt = (key >> shift) & 15;
+      const unsigned long long peers = digit_peers(valid, dgt);
       if (valid) {
-        const unsigned pos = sBinBase[dgt] + sOff[wave][dgt] + rank;
+        const unsigned pos = sCnt[wave][dgt] + __popcll(peers & ltMask);
         kDst[pos] = key;
         vDst[pos] = val;
       }
-      __syncthreads();
-      if (tid < 16) sBinBase[tid] += sTileTot[tid];
-      __syncthreads();
+      // the last peer moves the digit's running position (the wave's LDS accesses stay in order)
+      if (valid && (peers >> lane) == 1ull) sCnt[wave][dgt] += __popcll(peers);
     }
   }
 }
