@@ -86,9 +86,9 @@ def measured_traffic(args, sliced):
     workload and schedule it was measured on."""
     if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
         if sliced:
-            # slice_index + f3s_fwd_sliced + f3s_merge_slices
-            return (2 * (42_394 + 2_573_930 + 262_572) + 512 + 524_196 + 58_268) * 1024
-        return (2 * 7_350_110 + 58_241) * 1024
+            # slice_index_kernel + f3s_fwd_unit_kernel + f3s_merge_slices_kernel
+            return (2 * (42_398 + 2_635_240 + 262_572) + 512 + 524_196 + 58_269) * 1024
+        return (2 * 7_322_370 + 58_241) * 1024
     return None
 
 
