@@ -195,6 +195,108 @@ __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
   if (lane == 0) blockPartition[w] = (nUniq + W - 1) / W;
 }
 
+// The same job for graphs of at most 2^22 nodes, where a column id and the edge's position in
+// the window (< kSortMax = 2^10) fit one 32-bit word: a stable LSD radix sort of those words on
+// the column bits, eight bits per pass, in the wave's LDS slice (histogram with LDS atomics,
+// in-order scatter with wave ballots). The sorted words carry the edge positions along, so the
+// rank of every distinct column is scattered straight back to its edges: no binary search, and
+// a third of the instructions of the bitonic network.
+template <int W>
+__global__ __launch_bounds__(kBlock) void window_rank_radix_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int nRW,
+    int colBits, int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, int32_t* __restrict__ bigList) {
+  constexpr int WAVES = kBlock / 64;
+  constexpr int IDX_BITS = 10;
+  static_assert(kSortMax <= (1 << IDX_BITS), "edge position must fit IDX_BITS");
+  __shared__ uint32_t sBufA[WAVES][kSortMax];
+  __shared__ uint32_t sBufB[WAVES][kSortMax];
+  __shared__ __align__(16) uint32_t sHist[WAVES][256];
+  __shared__ int sRowW[WAVES][17];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int w = blockIdx.x * WAVES + wave;
+  if (w >= nRW) return;
+  const int r0 = w * 16;
+  int* sRow = sRowW[wave];
+  if (lane < 17) sRow[lane] = rowPtr[min(r0 + lane, N)];
+  wave_lds_sync();
+  const int eS = sRow[0], eE = sRow[16];
+  const int n = eE - eS;
+  if (n == 0) {
+    if (lane == 0) blockPartition[w] = 0;
+    return;
+  }
+  if (n > kSortMax) {  // left to window_rank_kernel, through the queue if there is one
+    if (bigList && lane == 0) bigList[atomicAdd(&hdr->nBig, 1)] = w;
+    return;
+  }
+  uint32_t* src = sBufA[wave];
+  uint32_t* dst = sBufB[wave];
+  uint32_t* hist = sHist[wave];
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  bool bad = false;
+  for (int i = lane; i < n; i += 64) {
+    uint32_t col = (uint32_t)colIdx[eS + i];
+    if (col >= (uint32_t)N) {
+      bad = true;
+      col = 0;
+    }
+    src[i] = (col << IDX_BITS) | (uint32_t)i;
+    edgeToRow[eS + i] = r0 + row_of_edge(sRow, eS + i);
+  }
+  if (bad) atomicOr(&hdr->error, 1);
+  for (int shift = IDX_BITS; shift < IDX_BITS + colBits; shift += 8) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) hist[lane + 64 * k] = 0;
+    wave_lds_sync();
+    for (int i = lane; i < n; i += 64) atomicAdd(&hist[(src[i] >> shift) & 255u], 1u);
+    wave_lds_sync();
+    {
+      // exclusive scan of the 256 counts: lane l owns bins 4l .. 4l+3
+      const uint4 c = reinterpret_cast<uint4*>(hist)[lane];
+      const unsigned sum = c.x + c.y + c.z + c.w;
+      const unsigned excl = wave_inclusive_scan(sum, lane) - sum;
+      reinterpret_cast<uint4*>(hist)[lane] =
+          make_uint4(excl, excl + c.x, excl + c.x + c.y, excl + c.x + c.y + c.z);
+    }
+    wave_lds_sync();
+    for (int base = 0; base < n; base += 64) {
+      const int i = base + lane;
+      const bool valid = i < n;
+      const uint32_t key = valid ? src[i] : 0u;
+      const unsigned dgt = (key >> shift) & 255u;
+      unsigned long long peers = __ballot(valid);
+#pragma unroll
+      for (int b = 0; b < 8; b++) {
+        const unsigned long long bal = __ballot((dgt >> b) & 1u);
+        peers &= ((dgt >> b) & 1u) ? bal : ~bal;
+      }
+      if (valid) dst[hist[dgt] + __popcll(peers & ltMask)] = key;
+      // the last peer advances the digit's position; the wave's LDS operations stay in order
+      if (valid && (peers >> lane) == 1ull) hist[dgt] += __popcll(peers);
+    }
+    wave_lds_sync();
+    uint32_t* t = src;
+    src = dst;
+    dst = t;
+  }
+  // ranks of the distinct columns, scattered to their edges
+  int nUniq = 0;
+  for (int base = 0; base < n; base += 64) {
+    const int i = base + lane;
+    const bool valid = i < n;
+    const uint32_t key = valid ? src[i] : 0u;
+    const bool first = valid && (i == 0 || (src[i - 1] >> IDX_BITS) != (key >> IDX_BITS));
+    const unsigned long long bal = __ballot(first);
+    if (valid)
+      edgeToColumn[eS + (int)(key & ((1u << IDX_BITS) - 1u))] =
+          nUniq + __popcll(bal & (ltMask | (1ull << lane))) - 1;
+    nUniq += __popcll(bal);
+  }
+  if (lane == 0) blockPartition[w] = (nUniq + W - 1) / W;
+}
+
 template <int W, int TB>
 __global__ __launch_bounds__(TB) void window_rank_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
@@ -677,14 +779,28 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
     const int smallGrid = (nRW + kBlock / 64 - 1) / (kBlock / 64);
     const bool big = (int64_t)E >= (int64_t)nRW * 2048;  // long windows on average
     int32_t* queue = big ? nullptr : valsTmp;
-    if (W == 16)
+    // short windows: radix sort of packed (column, position) words when the column ids leave
+    // room for the position, else the bitonic network on bare column ids
+    int colBits = 0;
+    while (colBits < 31 && ((int64_t)1 << colBits) < (int64_t)N) colBits++;
+    if (colBits <= 22) {
+      if (W == 16)
+        hipLaunchKernelGGL(window_rank_radix_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
+                           rowPtr, colIdx, N, nRW, colBits, blockPartition, edgeToColumn,
+                           edgeToRow, hdr, queue);
+      else
+        hipLaunchKernelGGL(window_rank_radix_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
+                           rowPtr, colIdx, N, nRW, colBits, blockPartition, edgeToColumn,
+                           edgeToRow, hdr, queue);
+    } else if (W == 16) {
       hipLaunchKernelGGL(window_rank_small_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
                          rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
                          queue);
-    else
+    } else {
       hipLaunchKernelGGL(window_rank_small_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
                          rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
                          queue);
+    }
     F3S_HIP_CHECK(hipGetLastError());
     // eight waves per window when windows are long (more loads and LDS atomics in flight)
 #define F3S_RANK(WW, TBB)                                                                     \

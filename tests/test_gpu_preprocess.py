@@ -96,6 +96,25 @@ def test_multi_pass_bitset_large_n(oracle_mod):
     compare_preprocess(got, want)
 
 
+def test_more_than_4m_nodes_takes_the_bitonic_short_window_kernel(oracle_mod):
+    """Above 2^22 nodes a column id and an edge position no longer share a 32-bit word, so short
+    windows are ranked by the bitonic kernel instead of the radix one; long windows (a hub row)
+    and the multi-pass bitset are in the same graph."""
+    print("case 5m_nodes", flush=True)
+    N = 5_000_011
+    rng = np.random.default_rng(11)
+    deg = np.zeros(N, np.int64)
+    rows = rng.choice(N, size=40_000, replace=False)
+    deg[rows] = rng.integers(1, 40, size=len(rows))
+    deg[123_456] = 3_000  # a window of more than 1024 edges
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(deg)
+    colIdx = rng.integers(0, N, size=int(rowPtr[-1])).astype(np.int32)  # unsorted, may repeat
+    got = run_gpu(rowPtr, colIdx, N)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
+    compare_preprocess(got, want)
+
+
 def test_empty_graph_and_tiny():
     print("case empty", flush=True)
     got = run_gpu(np.zeros(41, np.int32), np.zeros(0, np.int32), 40)
