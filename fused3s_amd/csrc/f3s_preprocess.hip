@@ -32,6 +32,7 @@ constexpr int kBlock = 256;
 constexpr int kRangeMax = 393216;  // columns per bitset pass: 48 KiB of bits + 12 KiB of prefixes
 constexpr int kSortMax = 1024;     // windows up to this many edges are ranked by a per-wave LDS sort
 constexpr int kFillChunk = 512;    // TC blocks held in LDS at once by window_fill_kernel
+constexpr int kFillChunkSmall = 128;  // the same for graphs of short windows (one wave each)
 
 // workspace header (bytes 0..255): int64 nTCB, int32 error flag, and the queue of windows too
 // long for the wave-per-window kernel (filled by window_rank_small_kernel, drained by
@@ -553,14 +554,13 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
 }
 
 // ------------------------------------------------------------------ phase 2
-template <int W, int TB>
+template <int W, int TB, int TC>
 __global__ __launch_bounds__(TB) void window_fill_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
     const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
     long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
     int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
-    unsigned long long* __restrict__ bitmap) {
-  constexpr int TC = kFillChunk;
+    unsigned long long* __restrict__ bitmap, int minBlocks, int maxBlocks) {
   constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
   constexpr int LOGW = (W == 16) ? 4 : 3;
   __shared__ unsigned sCnt[TC * 16];            // [block][row] counts, then running positions
@@ -577,7 +577,8 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
   if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
   const int base = rowWindowOffset[w];
   const int nb = rowWindowOffset[w + 1] - base;
-  if (nb == 0) return;
+  // a launch may be one of two that share the windows by length: [minBlocks, maxBlocks]
+  if (nb == 0 || nb < minBlocks || nb > maxBlocks) return;
   const int r0 = w * 16;
   if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
   __syncthreads();
@@ -844,17 +845,32 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
     return 0;
   }
   auto bm = reinterpret_cast<unsigned long long*>(bitmap);
-  // Windows with thousands of edges get 16 waves (one per row in the tile-id replay, 32 waves
-  // per CU to hide the latency of the LDS atomics and the ballot chains); short windows keep 4.
-#define F3S_FILL(WW, TBB)                                                                       \
-  hipLaunchKernelGGL((window_fill_kernel<WW, TBB>), dim3(nRW), dim3(TBB), 0, stream, rowPtr,   \
-                     colIdx, N, E, edgeToColumn, rowWindowOffset, (long long)nTcb, tcblockRowid, \
-                     tcblocktileId, tcblockOffset, sparseAToXidx, bm)
+  // Windows with thousands of edges get eight waves and 512 TC blocks of LDS at a time. Graphs
+  // of short windows get one wave per window and 128 blocks of LDS, so that a CU works on a
+  // dozen windows at once instead of three with most of their waves idle; their few windows of
+  // more than 128 blocks are left to a second launch with four waves per window.
+#define F3S_FILL(WW, TBB, TCC, LO, HI)                                                         \
+  hipLaunchKernelGGL((window_fill_kernel<WW, TBB, TCC>), dim3(nRW), dim3(TBB), 0, stream,      \
+                     rowPtr, colIdx, N, E, edgeToColumn, rowWindowOffset, (long long)nTcb,     \
+                     tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx, bm, LO, HI)
   const bool big = (int64_t)E >= (int64_t)nRW * 2048;
+  constexpr int kAll = 0x7FFFFFFF;
   if (W == 16) {
-    if (big) F3S_FILL(16, 512); else F3S_FILL(16, 256);
+    if (big) {
+      F3S_FILL(16, 512, kFillChunk, 0, kAll);
+    } else {
+      F3S_FILL(16, 64, kFillChunkSmall, 0, kFillChunkSmall);
+      F3S_HIP_CHECK(hipGetLastError());
+      F3S_FILL(16, 256, kFillChunk, kFillChunkSmall + 1, kAll);
+    }
   } else {
-    if (big) F3S_FILL(8, 512); else F3S_FILL(8, 256);
+    if (big) {
+      F3S_FILL(8, 512, kFillChunk, 0, kAll);
+    } else {
+      F3S_FILL(8, 64, kFillChunkSmall, 0, kFillChunkSmall);
+      F3S_HIP_CHECK(hipGetLastError());
+      F3S_FILL(8, 256, kFillChunk, kFillChunkSmall + 1, kAll);
+    }
   }
 #undef F3S_FILL
   F3S_HIP_CHECK(hipGetLastError());
