@@ -426,7 +426,10 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   constexpr int NW = kFinBlock / 64;
   __shared__ unsigned sWaveSum[NW];
   __shared__ int sWaveMax[NW];
-  __shared__ unsigned sCnt[NW][16];   // per wave: elements per digit, then its running position
+  constexpr int DB = 6;               // digit bits per sorting pass: one bin per lane
+  constexpr int NB = 1 << DB;
+  static_assert(NB == 64, "the start computation gives every lane one bin");
+  __shared__ unsigned sCnt[NW][NB];   // per wave: elements per digit, then its running position
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -476,29 +479,29 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   }
 
   // ---- stable sort by descending count == stable ascending LSD radix sort of (maxC - count),
-  // four bits per pass
+  // six bits per pass
   int nBits = 0;
   while ((maxC >> nBits) != 0) nBits++;
-  const int nPass = (nBits + 3) / 4;
+  const int nPass = (nBits + DB - 1) / DB;
   if (nPass == 0) {
     for (int i = tid; i < nRW; i += kFinBlock) sortedRowWindows[i] = i;
     return;
   }
   const unsigned long long ltMask = (1ull << lane) - 1ull;
   for (int pass = 0; pass < nPass; pass++) {
-    const int shift = pass * 4;
+    const int shift = pass * DB;
     const bool toOut = ((nPass - 1 - pass) & 1) == 0;
     int32_t* kDst = toOut ? keysA : keysB;
     int32_t* vDst = toOut ? sortedRowWindows : valsTmp;
     const int32_t* kSrc = toOut ? keysB : keysA;
     const int32_t* vSrc = toOut ? valsTmp : sortedRowWindows;
     __syncthreads();  // the previous pass's writes are visible, its use of sCnt is over
-    if (lane < 16) sCnt[wave][lane] = 0;
-    // peers = lanes of this 64-element group with the same digit (four ballots)
+    sCnt[wave][lane] = 0;
+    // peers = lanes of this 64-element group with the same digit (one ballot per digit bit)
     auto digit_peers = [&](bool valid, int dgt) {
       unsigned long long peers = __ballot(valid);
 #pragma unroll
-      for (int b = 0; b < 4; b++) {
+      for (int b = 0; b < DB; b++) {
         const unsigned long long bal = __ballot((dgt >> b) & 1);
         peers &= ((dgt >> b) & 1) ? bal : ~bal;
       }
@@ -515,22 +518,22 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
       const bool valid = i < cEnd;
       const int key = keyNext;
       keyNext = load_key(i + 64);
-      const int dgt = (key >> shift) & 15;
+      const int dgt = (key >> shift) & (NB - 1);
       const unsigned long long peers = digit_peers(valid, dgt);
       if (valid && (peers & ltMask) == 0ull) sCnt[wave][dgt] += __popcll(peers);
     }
     __syncthreads();
-    // start of (digit, wave): all smaller digits, then the same digit in earlier waves
-    unsigned start = 0;
-    if (lane < 16) {
-      for (int d2 = 0; d2 < 16; d2++)
-        for (int k = 0; k < NW; k++) {
-          const unsigned cnt = sCnt[k][d2];
-          if (d2 < lane || (d2 == lane && k < wave)) start += cnt;
-        }
+    // start of (digit = lane, wave): all smaller digits, then the same digit in earlier waves
+    unsigned digitTotal = 0, before = 0;
+#pragma unroll
+    for (int k = 0; k < NW; k++) {
+      const unsigned cnt = sCnt[k][lane];
+      digitTotal += cnt;
+      if (k < wave) before += cnt;
     }
+    const unsigned start = wave_inclusive_scan(digitTotal, lane) - digitTotal + before;
     __syncthreads();
-    if (lane < 16) sCnt[wave][lane] = start;
+    sCnt[wave][lane] = start;
     // scatter, in order
     keyNext = load_key(cBegin + lane);
     int valNext = load_val(cBegin + lane);
@@ -540,7 +543,7 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
       const int key = keyNext, val = valNext;
       keyNext = load_key(i + 64);
       valNext = load_val(i + 64);
-      const int dgt = (key >> shift) & 15;
+      const int dgt = (key >> shift) & (NB - 1);
       const unsigned long long peers = digit_peers(valid, dgt);
       if (valid) {
         const unsigned pos = sCnt[wave][dgt] + __popcll(peers & ltMask);
