@@ -655,6 +655,28 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
         unsigned run = carry + waveOff + incl - nnz;
         tcblockOffset[gt] = (int)run;
         tcblockRowid[gt] = w;
+        if (sUnsorted == 0u) {
+          // Every row of the window is strictly ascending, so the block's tile ids are its set
+          // bits read row by row, left to right (src/utils.cu:213-223 walks the edges in that
+          // order): this thread writes them all, next to the previous block's.
+          unsigned long long words[WPT];
+#pragma unroll
+          for (int k = 0; k < WPT; k++) words[k] = sBm[t * WPT + k];
+          unsigned pos = run;
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            unsigned rowBits = 0;  // W bits, column 0 in the most significant one
+#pragma unroll
+            for (int h = 0; h < W / 8; h++)
+              rowBits = (rowBits << 8) |
+                        ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
+            while (rowBits) {
+              const int cl = __clz(rowBits) - (32 - W);
+              tcblocktileId[pos++] = (uint8_t)(r * W + cl);
+              rowBits &= ~(1u << (W - 1 - cl));
+            }
+          }
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const unsigned c = sCnt[t * 16 + r];
@@ -684,12 +706,13 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
       carry += tileTot;
       __syncthreads();
     }
-    // Tile ids sit in CSR edge order inside a TC block (src/utils.cu:213-223): position =
-    // start of (block, row) + number of earlier edges of that row in the block. In a strictly
-    // ascending row those are exactly the bits left of the edge's own bit in the block's bitmap
-    // row, so every edge finds its place on its own.
+    // Windows with some row that is not strictly ascending. Tile ids sit in CSR edge order
+    // inside a TC block (src/utils.cu:213-223): position = start of (block, row) + number of
+    // earlier edges of that row in the block. In a strictly ascending row those are exactly the
+    // bits left of the edge's own bit in the block's bitmap row, so every edge of such a row
+    // finds its place on its own; the other rows are replayed in order below.
     const unsigned unsorted = sUnsorted;
-    for (int e = eS + tid; e < eE; e += TB) {
+    for (int e = eS + tid; unsorted != 0u && e < eE; e += TB) {
       const int ec = edgeToColumn[e];
       const int t = (ec >> LOGW) - tc0;
       if ((unsigned)t >= (unsigned)nt) continue;
