@@ -87,8 +87,8 @@ def measured_traffic(args, sliced):
     if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
         if sliced:
             # slice_index_kernel + f3s_fwd_unit_kernel + f3s_merge_slices_kernel
-            return (2 * (42_398 + 2_635_240 + 262_572) + 512 + 524_196 + 58_269) * 1024
-        return (2 * 7_322_370 + 58_241) * 1024
+            return (2 * (42_397 + 2_642_050 + 262_572) + 512 + 524_196 + 58_270) * 1024
+        return (2 * 7_353_770 + 58_241) * 1024
     return None
 
 
