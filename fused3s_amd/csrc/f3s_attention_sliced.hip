@@ -1,19 +1,23 @@
-// Fused 3S attention, column-sliced schedule (gfx950). Same arithmetic per TC-block pair as
-// f3s_fwd_kernel (f3s_attention.hip, which documents the register dataflow and the numerics);
-// what differs is the decomposition:
+// Fused 3S attention with one wave per unit of work (gfx950). Same arithmetic per TC-block pair
+// as f3s_fwd_kernel (f3s_attention.hip, which documents the register dataflow and the numerics);
+// what differs is the decomposition. Two uses of the one kernel, f3s_fwd_unit_kernel:
 //
+// Column-sliced schedule, for graphs with long windows:
 //   * the column range is cut into S = 8 * P slices. Workgroup b runs on XCD b % 8 (the hardware
 //     deals workgroups round-robin over the eight XCDs), and the grid is laid out so that XCD x
 //     only ever works on slices x, x + 8, x + 16, ..., one after the other. The K/V rows of a
-//     slice fit in the XCD's 4 MiB L2, so a row is fetched from the memory side once per XCD
-//     instead of once per window that names it;
+//     slice mostly stay in the XCD's 4 MiB L2, so a row is fetched from the memory side about
+//     once per XCD instead of once per window that names it;
 //   * a wave computes one (window, slice) unit: the window's TC blocks whose first column falls
 //     into the slice, with (m, l, O) in registers, and writes the unit's partial result to
 //     scratch. A second kernel merges a window's partials (log-sum-exp) and writes its rows.
 //
+// Wave per window, for graphs of short windows: a unit is a whole window (of one head); the rows
+// are written straight from the registers.
+//
 // The reference has no counterpart: its kernels (src/F3S_kernel.cu:1371-1583) walk one window
 // per thread block from its first TC block to its last. Its window order (src/utils.cu:400-436)
-// is kept: units are issued heavy windows first inside every slice.
+// is kept: units are issued heavy windows first.
 #include <stdlib.h>
 
 #include "f3s_common.h"

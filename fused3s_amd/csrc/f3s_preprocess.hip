@@ -4,23 +4,27 @@
 // a global thrust::sort of (window, column) pairs followed by two kernels that walk each
 // window with a single thread. Here a window never leaves its workgroup:
 //
-//   window_rank_small_kernel  windows of <= 1024 edges, one WAVE per window: bitonic sort of the
-//                        column ids in LDS, ballot / popcount compaction of the distinct ones,
-//                        rank by binary search. No workgroup barrier.
+//   window_rank_radix_kernel / window_rank_small_kernel
+//                        windows of <= 1024 edges, one WAVE per window, no workgroup barrier.
+//                        Graphs of <= 2^22 nodes: stable LSD radix sort of (column, position)
+//                        words in LDS, ranks of the distinct columns scattered back to the
+//                        edges. Larger graphs: bitonic sort of the column ids, ballot / popcount
+//                        compaction of the distinct ones, rank by binary search.
 //   window_rank_kernel   larger windows, one workgroup per window. Column ids are OR-ed into an
-//                        LDS bitset
-//                        (a column range per pass when N exceeds the LDS range), a wave64
-//                        popcount prefix scan turns the bitset into ranks, and every edge
+//                        LDS bitset (a column range per pass when N exceeds the LDS range), a
+//                        wave64 popcount prefix scan turns the bitset into ranks, and every edge
 //                        reads its compacted column index back: the sorted unique column list
 //                        (reference: sort + inplace_deduplication + binarysearch,
 //                        src/utils.cu:102-153,281-289) is never materialised.
-//   finalize_count_kernel one workgroup: inclusive scan of the per-window block counts
-//                        (src/utils.cu:293-300) and a stable LSD radix sort of the windows by
-//                        descending block count (src/utils.cu:400-436), ranks from wave ballots.
-//   window_fill_kernel   one workgroup per window: bitmaps and per-(row, block) edge counts are
-//                        accumulated in LDS, a block-wide scan yields the per-block offsets, and
-//                        each wave replays its rows in CSR order to place the tile ids
-//                        (src/utils.cu:173-224, 23-36, 53-65).
+//   finalize_count_kernel one workgroup, every wave on its own chunk of the windows: inclusive
+//                        scan of the per-window block counts (src/utils.cu:293-300) and a stable
+//                        LSD radix sort of the windows by descending block count
+//                        (src/utils.cu:400-436), ranks from wave ballots.
+//   window_fill_kernel   one workgroup (or one wave, on graphs of short windows) per window:
+//                        bitmaps and per-(row, block) edge counts are accumulated in LDS, a scan
+//                        yields the per-block offsets, and the tile ids are written per block
+//                        from its bitmap when the window's rows ascend, else placed edge by edge
+//                        in CSR order (src/utils.cu:173-224, 23-36, 53-65).
 //
 // All results are bit-identical to the reference's algorithm with edgeToRow[e] = row(e).
 #include "f3s_common.h"
