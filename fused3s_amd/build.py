@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libf3s_amd.so")
 EXT_PATH = os.path.join(HERE, "F3S" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
-HIP_SOURCES = ["f3s_capi.hip", "f3s_attention.hip", "f3s_attention_sliced.hip", "f3s_preprocess.hip"]
+HIP_SOURCES = ["f3s_capi.hip", "f3s_attention.hip", "f3s_attention_units.hip", "f3s_preprocess.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall",
     # packed-fp32 code generation is switched off for every device translation unit

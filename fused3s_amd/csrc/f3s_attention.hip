@@ -517,7 +517,7 @@ bool split_short_windows(const int32_t* windowOrder, int nRW, int64_t nTcb, Head
   return true;
 }
 
-// The column-sliced schedule (f3s_attention_sliced.hip: (window, column slice) units, every XCD
+// The column-sliced schedule (f3s_attention_units.hip: (window, column slice) units, every XCD
 // on one slice at a time so that its K/V rows stay in that XCD's L2, plus a merge kernel) pays off
 // on graphs with long windows: on the 233k-node benchmark graph (475 TC blocks per window) it
 // takes 1.66 / 1.94 / 3.67 ms at d = 32 / 64 / 128 against 2.27 / 2.11 / 6.05 ms for the

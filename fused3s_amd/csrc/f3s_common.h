@@ -41,7 +41,7 @@ int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowO
 
 int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype);
 
-// column-sliced schedule (f3s_attention_sliced.hip)
+// column-sliced schedule (f3s_attention_units.hip)
 size_t attention_sliced_workspace_bytes(int N, int d);
 int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                             const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
