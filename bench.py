@@ -79,6 +79,38 @@ def cpu_baseline(rowPtr, colIdx, N, Q, K, V, scale, d, budget_s=12.0):
                       "(%d rows, %d edges), %.1f s wall" % (step, rows_done, edges, spent)}
 
 
+def cpu_baseline_torch(rowPtr, colIdx, N, Q, K, V, scale, d, max_edges=4_000_000):
+    """The reference's own CPU formulation of the computation, edge-wise SDDMM -> segment softmax
+    -> SpMM with plain PyTorch ops (scripts/baseline_comp/baseline_comp_kernel_only.py:667-686
+    does it with PyG's softmax / scatter; PyG is not installed here, so index_add_ / index_reduce_
+    stand in), fp32 on the host cores, on the first rows of the graph up to max_edges edges."""
+    rp = rowPtr.cpu().long()
+    rows_n = int(torch.searchsorted(rp, torch.tensor(max_edges)).clamp(min=1, max=N))
+    e = int(rp[rows_n])
+    if e == 0:
+        return None
+    col = colIdx[:e].cpu().long()
+    row = torch.repeat_interleave(torch.arange(rows_n), rp[1:rows_n + 1] - rp[:rows_n])
+    Qf, Kf, Vf = (x.float().cpu() for x in (Q, K, V))
+    torch.set_num_threads(os.cpu_count() or 1)
+
+    def run():
+        s_e = (Qf[row] * Kf[col]).sum(-1) / scale
+        mx = torch.full((rows_n,), float("-inf")).index_reduce_(0, row, s_e, "amax")
+        p = torch.exp(s_e - mx[row])
+        den = torch.zeros(rows_n).index_add_(0, row, p)
+        out = torch.zeros((rows_n, d)).index_add_(0, row, (p / den[row]).unsqueeze(1) * Vf[col])
+        return out
+    run()
+    t0 = time.time()
+    run()
+    dt = time.time() - t0
+    return {"value": 4.0 * d * e / dt / 1e12, "unit": "TFLOP/s (effective, 4*d*E/t)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "edge-wise PyTorch CPU ops (gather, index_reduce_, index_add_) on the first "
+                      "%d rows (%d edges), %.2f s" % (rows_n, e, dt)}
+
+
 def measured_traffic(args, sliced):
     """HBM-side bytes per attention call from rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
     factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md). Counters cannot
@@ -264,6 +296,8 @@ def main():
         result["cpu_baseline"] = cpu_baseline(rowPtr, colIdx, N, q1, k1, v1, scale, d,
                                               args.cpu_budget)
         log("cpu baseline:", result["cpu_baseline"])
+        result["cpu_baseline_torch"] = cpu_baseline_torch(rowPtr, colIdx, N, q1, k1, v1, scale, d)
+        log("cpu baseline (PyTorch ops):", result["cpu_baseline_torch"])
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result), flush=True)
