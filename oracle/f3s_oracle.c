@@ -156,47 +156,59 @@ int64_t f3s_oracle_preprocess_count(const int32_t *rowPtr, const int32_t *colIdx
                                     int32_t *rowWindowOffset) {
   int nRW = (N + H - 1) / H;
   int64_t total = 0;
-  int32_t *tmp = NULL;
-  int64_t cap = 0;
-  for (int w = 0; w < nRW; w++) {
-    int64_t s = rowPtr[(int64_t)w * H];
-    int64_t e = rowPtr[imin(w * H + H, N)];
-    int64_t n = e - s;
-    if (n == 0) continue;
-    if (n > cap) {
-      free(tmp);
-      cap = n * 2;
-      tmp = (int32_t *)malloc(sizeof(int32_t) * (size_t)cap);
-      if (!tmp) return -1;
-    }
-    memcpy(tmp, colIdx + s, sizeof(int32_t) * (size_t)n);
-    qsort(tmp, (size_t)n, sizeof(int32_t), cmp_i32);
-    int64_t loc = 0; /* index of the last unique element, as in inplace_deduplication */
-    for (int64_t cur = 1; cur < n; cur++) {
-      if (tmp[cur] != tmp[cur - 1]) tmp[++loc] = tmp[cur];
-    }
-    int num = (int)((loc + W) / W);
-    blockPartition[w] = num;
-    total += num;
-    for (int64_t k = s; k < e; k++) {
-      int32_t target = colIdx[k];
-      int64_t lo = 0, hi = loc;
-      int64_t idx = -1;
-      while (lo <= hi) {
-        int64_t mid = lo + (hi - lo) / 2;
-        if (tmp[mid] == target) {
-          idx = mid;
-          break;
+  int failed = 0;
+  /* windows are independent of each other (the reference handles one per thread,
+   * src/utils.cu:131-153), so they are shared out over the host cores */
+#pragma omp parallel reduction(+ : total)
+  {
+    int32_t *tmp = NULL;
+    int64_t cap = 0;
+#pragma omp for schedule(dynamic, 16)
+    for (int w = 0; w < nRW; w++) {
+      int64_t s = rowPtr[(int64_t)w * H];
+      int64_t e = rowPtr[imin(w * H + H, N)];
+      int64_t n = e - s;
+      if (n == 0) continue;
+      if (n > cap) {
+        free(tmp);
+        cap = n * 2;
+        tmp = (int32_t *)malloc(sizeof(int32_t) * (size_t)cap);
+        if (!tmp) {
+          cap = 0;
+          failed = 1;
+          continue;
         }
-        if (tmp[mid] < target)
-          lo = mid + 1;
-        else
-          hi = mid - 1;
       }
-      edgeToColumn[k] = (int32_t)idx;
+      memcpy(tmp, colIdx + s, sizeof(int32_t) * (size_t)n);
+      qsort(tmp, (size_t)n, sizeof(int32_t), cmp_i32);
+      int64_t loc = 0; /* index of the last unique element, as in inplace_deduplication */
+      for (int64_t cur = 1; cur < n; cur++) {
+        if (tmp[cur] != tmp[cur - 1]) tmp[++loc] = tmp[cur];
+      }
+      int num = (int)((loc + W) / W);
+      blockPartition[w] = num;
+      total += num;
+      for (int64_t k = s; k < e; k++) {
+        int32_t target = colIdx[k];
+        int64_t lo = 0, hi = loc;
+        int64_t idx = -1;
+        while (lo <= hi) {
+          int64_t mid = lo + (hi - lo) / 2;
+          if (tmp[mid] == target) {
+            idx = mid;
+            break;
+          }
+          if (tmp[mid] < target)
+            lo = mid + 1;
+          else
+            hi = mid - 1;
+        }
+        edgeToColumn[k] = (int32_t)idx;
+      }
     }
+    free(tmp);
   }
-  free(tmp);
+  if (failed) return -1;
   rowWindowOffset[0] = 0;
   for (int w = 0; w < nRW; w++) rowWindowOffset[w + 1] = rowWindowOffset[w] + blockPartition[w];
   return total;
@@ -215,6 +227,7 @@ int64_t f3s_oracle_preprocess_count(const int32_t *rowPtr, const int32_t *colIdx
 void f3s_oracle_fill_edge_to_row(const int32_t *rowPtr, int N, int emulate_stride_bug,
                                  int32_t *edgeToRow) {
   if (!emulate_stride_bug) {
+#pragma omp parallel for schedule(static)
     for (int r = 0; r < N; r++)
       for (int64_t k = rowPtr[r]; k < rowPtr[r + 1]; k++) edgeToRow[k] = r;
     return;
@@ -268,6 +281,8 @@ void f3s_oracle_preprocess_fill(const int32_t *rowPtr, const int32_t *colIdx, in
   memset(bitmap, 0, sizeof(uint64_t) * (size_t)(nTCB * wordsPerTcb));
   memset(tcblockOffset, 0, sizeof(int32_t) * (size_t)(nTCB + 1));
   memset(tcblocktileId, 0, (size_t)E);
+  /* a window only writes its own TC blocks and its own edges: shared out over the host cores */
+#pragma omp parallel for schedule(dynamic, 16)
   for (int w = 0; w < nRW; w++) {
     int64_t base = rowWindowOffset[w];
     int64_t nb = rowWindowOffset[w + 1] - base;
@@ -337,8 +352,9 @@ static inline int tcb_bit(const uint64_t *bitmap, int64_t t, int rl, int cl) {
  * The window order is irrelevant to the result (windows are independent), so the
  * sortedRowWindows argument of the reference is not needed here.
  * Rows >= N of the last window are treated as all-zero Q and never written.
- * dtype: 0 = fp16 inputs (the reference), 1 = bf16 inputs (beyond the reference: same
- * algorithm with P rounded to bf16, the type both operands of a bf16 matrix product share).
+ * dtype: 0 = fp16 inputs (the reference), 1 = bf16 inputs (beyond the reference, which is
+ * fp16-only, src/F3S_kernel.cu:622-624): the same algorithm on the bf16 values, with P still
+ * rounded to fp16 as the reference rounds it (:938-945).
  */
 int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *sparseAToXidx,
                              const uint64_t *bitmap, int N, int d, int dtype, const uint16_t *Q,
@@ -393,13 +409,13 @@ int f3s_oracle_attention_ref(const int32_t *rowWindowOffset, const int32_t *spar
             for (int i = 0; i < nb * 16; i++) {
               float ev = (S[i] == 0.0f) ? 0.0f : expf(S[i] - mnew);
               sum += ev;
-              P[i] = dtype == 0 ? round_to_half(ev) : round_to_bf16(ev);
+              P[i] = round_to_half(ev);
             }
             l = fmaf(alpha, l, sum);
             for (int c = 0; c < d; c++) O[c] *= alpha;
           } else {
             for (int i = 0; i < nb * 16; i++)
-              P[i] = dtype == 0 ? round_to_half(S[i]) : round_to_bf16(S[i]);
+              P[i] = round_to_half(S[i]);
           }
           for (int b = 0; b < nb; b++) {
             for (int j = 0; j < 16; j++) {

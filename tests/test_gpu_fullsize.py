@@ -1,13 +1,43 @@
-"""The benchmark graphs at full size, checked through properties that need no full CPU run:
-a bounded sample of rows against the textbook oracle, softmax weights summing to one, agreement of
-the two window orders and of the two schedules, and preprocessing invariants."""
+"""The benchmark graphs at full size: preprocessing bit-exact against the CPU oracle on every
+output, the fused attention on ALL rows against the reference-emulating oracle (max-abs 2e-2 /
+mean-relative 1e-3) for both schedules, plus properties that need no CPU run (softmax weights
+summing to one, agreement of the two window orders, preprocessing invariants) and a bounded sample
+of rows against the textbook oracle."""
 import numpy as np
 import pytest
 import torch
 
+from ref_checks import compare_preprocess
+
 pytestmark = pytest.mark.gpu
 MAX_ABS = 2e-2
 MEAN_REL = 1e-3
+
+
+def host(res):
+    out = {}
+    for k, v in res.items():
+        if torch.is_tensor(v):
+            v = v.cpu()
+            out[k] = v.view(torch.int64).numpy().view(np.uint64) if v.dtype == torch.uint64 \
+                else v.numpy()
+        else:
+            out[k] = v
+    return out
+
+
+def bits16(t):
+    """fp16 / bf16 device tensor -> numpy array the oracle takes (float16, or uint16 bits)."""
+    t = t.contiguous().cpu()
+    return t.numpy() if t.dtype == torch.float16 else t.view(torch.int16).numpy().view(np.uint16)
+
+
+def check_close(got, want, what):
+    err = float(np.abs(got - want).max())
+    rel = float(np.abs(got - want).mean() / max(np.abs(want).mean(), 1e-30))
+    print("  %s: max-abs %.2e mean-rel %.2e" % (what, err, rel), flush=True)
+    assert err < MAX_ABS, (what, err)
+    assert rel < MEAN_REL, (what, rel)
 
 
 @pytest.mark.parametrize("name", ["cfg3_chunglu_233k", "cfg4_rmat_2449k"])
@@ -23,6 +53,14 @@ def test_full_size_graph(oracle_mod, name):
     pre = capi.preprocess(rowPtr, colIdx, N)
     nT = pre["blockCount"]
     rwo = pre["rowWindowOffset"]
+
+    # every preprocessing output, bit for bit, against the CPU oracle at full size
+    rp, ci = rowPtr.cpu().numpy(), colIdx.cpu().numpy()
+    want_pre = oracle_mod.preprocess(rp, ci, N)
+    compare_preprocess(host(pre), want_pre)
+    for k in ("tcblocktileId", "tcblockOffset", "tcblockRowid", "edgeToColumn", "edgeToRow",
+              "blockPartition"):
+        del want_pre[k]
 
     # preprocessing invariants (scripts/graph_stat/paper_graph_stat.py:68-72 and the bitmap's
     # definition): per-block non-zeros add up to E, one bit per distinct (row, column) pair,
@@ -52,16 +90,25 @@ def test_full_size_graph(oracle_mod, name):
     torch.cuda.synchronize()
     assert bool(torch.isfinite(out).all())
 
+    # all rows against the reference-emulating oracle
+    Qh, Kh, Vh = Q.cpu().numpy(), K.cpu().numpy(), V.cpu().numpy()
+    ref = oracle_mod.attention_ref(want_pre["rowWindowOffset"], want_pre["sparseAToXidx"],
+                                   want_pre["tcbBitMap"], N, Qh, Kh, Vh, scale)
+    check_close(out.cpu().numpy(), ref, "%s window schedule vs attention_ref" % name)
+
     # both window orders give the same rows, bit for bit (same arithmetic per window)
     nat = capi.attention(rwo, None, *args[2:])
     assert torch.equal(nat, out)
+    del nat
 
     # the column-sliced schedule (used when the library judges the graph dense enough)
     ws = capi.attention_workspace(N, d, dev, nTCB=nT)
     if ws is not None:
         sl = capi.attention(*args, workspace=ws)
+        check_close(sl.cpu().numpy(), ref, "%s column-sliced schedule vs attention_ref" % name)
         assert float((sl - out).abs().max()) < 2e-3
         del sl, ws
+    del ref
 
     # softmax weights sum to one: with V = 1 every row with an edge gives exactly ~1, others 0
     ones = torch.ones_like(V)
@@ -74,10 +121,62 @@ def test_full_size_graph(oracle_mod, name):
 
     # a bounded, evenly spaced sample of rows against the textbook oracle
     step = max(1, N // 1500)
-    rp, ci = rowPtr.cpu().numpy(), colIdx.cpu().numpy()
-    want = oracle_mod.attention_textbook(rp, ci, N, Q.cpu().numpy(), K.cpu().numpy(),
-                                         V.cpu().numpy(), scale, row_step=step)
+    want = oracle_mod.attention_textbook(rp, ci, N, Qh, Kh, Vh, scale, row_step=step)
     sel = np.arange(0, N, step)
     got = out[torch.as_tensor(sel, device=dev)].cpu().numpy()
     assert np.abs(got - want[sel]).max() < MAX_ABS
     assert np.abs(got - want[sel]).mean() / np.abs(want[sel]).mean() < MEAN_REL
+
+
+def test_config2_attention_full_size(oracle_mod):
+    """169k-node R-MAT graph, d = 64 fp16: the fused attention on its own workload, all rows,
+    heavy-first and natural order, against the reference-emulating oracle."""
+    from fused3s_amd import capi, synth
+    print("case fullsize attention cfg2_rmat_169k", flush=True)
+    dev = torch.device("cuda:0")
+    rowPtr, colIdx = synth.make_graph("cfg2_rmat_169k", seed=0, device=dev)
+    N = rowPtr.numel() - 1
+    pre = capi.preprocess(rowPtr, colIdx, N)
+    Q, K, V = synth.features(N, 64, seed=0, device=dev)
+    hp = host(pre)
+    ref = oracle_mod.attention_ref(hp["rowWindowOffset"], hp["sparseAToXidx"], hp["tcbBitMap"], N,
+                                   bits16(Q), bits16(K), bits16(V), 8.0)
+    for order in (pre["sortedRowWindows"], None):
+        out = capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
+                             pre["tcbBitMap"], N, Q, K, V, 8.0)
+        check_close(out.cpu().numpy(), ref, "cfg2 %s order" % ("natural" if order is None
+                                                              else "heavy-first"))
+    txt = oracle_mod.attention_textbook(rowPtr.cpu().numpy(), colIdx.cpu().numpy(), N, bits16(Q),
+                                        bits16(K), bits16(V), 8.0)
+    check_close(out.cpu().numpy(), txt, "cfg2 vs textbook")
+
+
+@pytest.mark.parametrize("name", ["cfg5_sbm_100k", "cfg5b_sbm_100k_dense"])
+def test_config5_multihead_layer_full_size(oracle_mod, name):
+    """100k-node block-model graph (p_in = 0.02 as stated, and 0.2 for the stated edge count),
+    8 heads x d = 32 bf16 through f3s_attention_fwd_heads: every head against the
+    reference-emulating oracle run on that head's bf16 values (P rounded to fp16 as the reference
+    rounds it), at the stated tolerance."""
+    from fused3s_amd import capi, synth
+    print("case fullsize heads %s" % name, flush=True)
+    dev = torch.device("cuda:0")
+    cfg = synth.CONFIGS[name]
+    H, d = cfg["heads"], cfg["d"]
+    rowPtr, colIdx = synth.make_graph(name, seed=0, device=dev)
+    N = rowPtr.numel() - 1
+    pre = capi.preprocess(rowPtr, colIdx, N)
+    hp = host(pre)
+    compare_preprocess(hp, oracle_mod.preprocess(rowPtr.cpu().numpy(), colIdx.cpu().numpy(), N))
+    Q, K, V = synth.features(N, H * d, seed=0, device=dev, dtype=torch.bfloat16, std=d ** -0.5)
+    Q, K, V = (x.view(N, H, d) for x in (Q, K, V))
+    scale = float(np.sqrt(d))
+    out = capi.attention_heads(pre["rowWindowOffset"], pre["sortedRowWindows"],
+                               pre["sparseAToXidx"], pre["tcbBitMap"], N, Q, K, V, scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert got.shape == (N, H * d)
+    for h in range(H):
+        ref = oracle_mod.attention_ref(hp["rowWindowOffset"], hp["sparseAToXidx"], hp["tcbBitMap"],
+                                       N, bits16(Q[:, h]), bits16(K[:, h]), bits16(V[:, h]), scale,
+                                       dtype=1)
+        check_close(got[:, h * d:(h + 1) * d], ref, "%s head %d" % (name, h))
