@@ -16,7 +16,8 @@ _lib = None
 EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes",
            "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
            "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads",
-           "f3s_attention_fwd_tcb8", "f3s_attention_uses_workspace"]
+           "f3s_attention_fwd_tcb8", "f3s_attention_uses_workspace",
+           "f3s_preprocess_static_scratch_bytes", "f3s_preprocess_count_static"]
 
 
 def lib():
@@ -34,6 +35,11 @@ def lib():
         L.f3s_preprocess_count.restype = ci
         L.f3s_preprocess_count.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, cs,
                                            ctypes.POINTER(ctypes.c_int64), vp]
+        L.f3s_preprocess_static_scratch_bytes.restype = cs
+        L.f3s_preprocess_static_scratch_bytes.argtypes = []
+        L.f3s_preprocess_count_static.restype = ci
+        L.f3s_preprocess_count_static.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp,
+                                                  vp]
         L.f3s_preprocess_fill.restype = ci
         L.f3s_preprocess_fill.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, ctypes.c_int64, vp, vp,
                                           vp, vp, vp, vp]
@@ -112,6 +118,25 @@ def preprocess(rowPtr, colIdx, N, H=16, W=16):
                 tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox, tcbBitMap=bm,
                 blockCount=nT, blockPartition=blockPartition, edgeToColumn=edgeToColumn,
                 edgeToRow=edgeToRow)
+
+
+def preprocess_count_static(rowPtr, colIdx, N, out, H=16, W=16):
+    """f3s_preprocess_count_static on the current stream: phase 1 with the library's own scratch
+    and no host round trip. `out` holds caller-allocated device tensors blockPartition,
+    edgeToColumn, edgeToRow, rowWindowOffset, sortedRowWindows (int32) and result (int64[2]:
+    TC-block total, error flag); nothing is allocated here."""
+    L = lib()
+    _dev(rowPtr, torch.int32, "rowPtr")
+    _dev(colIdx, torch.int32, "colIdx")
+    for name in ("blockPartition", "edgeToColumn", "edgeToRow", "rowWindowOffset",
+                 "sortedRowWindows"):
+        _dev(out[name], torch.int32, name)
+    _dev(out["result"], torch.int64, "result")
+    with torch.cuda.device(rowPtr.device):
+        _check(L.f3s_preprocess_count_static(
+            _ptr(rowPtr), _ptr(colIdx), N, int(colIdx.numel()), H, W, _ptr(out["blockPartition"]),
+            _ptr(out["edgeToColumn"]), _ptr(out["edgeToRow"]), _ptr(out["rowWindowOffset"]),
+            _ptr(out["sortedRowWindows"]), _ptr(out["result"]), _stream()))
 
 
 def attention_workspace(N, d, device, nTCB=None, dtype=torch.float16):

@@ -52,6 +52,26 @@ int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, in
                                       ws_bytes, nTCB_host, static_cast<hipStream_t>(stream));
 }
 
+size_t f3s_preprocess_static_scratch_bytes(void) { return f3s::preprocess_static_scratch_bytes(); }
+
+int f3s_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                                int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                                int32_t* edgeToRow, int32_t* rowWindowOffset,
+                                int32_t* sortedRowWindows, int64_t* result_dev, void* stream) {
+  if (!rowPtr || !rowWindowOffset || !result_dev)
+    return f3s::fail(-1, "f3s_preprocess_count_static: null pointer");
+  if (N > 0 && (!blockPartition || !sortedRowWindows))
+    return f3s::fail(-1, "f3s_preprocess_count_static: null window output");
+  if (E > 0 && (!colIdx || !edgeToColumn || !edgeToRow))
+    return f3s::fail(-1, "f3s_preprocess_count_static: null edge array");
+  if (f3s::misaligned(result_dev, 8))
+    return f3s::fail(-1, "f3s_preprocess_count_static: result_dev must be 8-byte aligned");
+  return f3s::launch_preprocess_count_static(rowPtr, colIdx, N, E, H, W, blockPartition,
+                                             edgeToColumn, edgeToRow, rowWindowOffset,
+                                             sortedRowWindows, result_dev,
+                                             static_cast<hipStream_t>(stream));
+}
+
 int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
                         const int32_t* edgeToColumn, const int32_t* rowWindowOffset, int64_t nTCB,
                         int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,

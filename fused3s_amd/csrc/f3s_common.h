@@ -63,6 +63,12 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
                             int32_t* edgeToRow, int32_t* rowWindowOffset,
                             int32_t* sortedRowWindows, void* workspace, size_t wsBytes,
                             int64_t* nTcbHost, hipStream_t stream);
+size_t preprocess_static_scratch_bytes();
+int launch_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, int N, int E,
+                                   int H, int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                                   int32_t* edgeToRow, int32_t* rowWindowOffset,
+                                   int32_t* sortedRowWindows, int64_t* resultDev,
+                                   hipStream_t stream);
 int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
                            int W, const int32_t* edgeToColumn, const int32_t* rowWindowOffset,
                            int64_t nTcb, int32_t* tcblockRowid, uint8_t* tcblocktileId,

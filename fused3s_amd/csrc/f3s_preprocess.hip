@@ -27,7 +27,15 @@
 //                        in CSR order (src/utils.cu:173-224, 23-36, 53-65).
 //
 // All results are bit-identical to the reference's algorithm with edgeToRow[e] = row(e).
+#include <mutex>
+
 #include "f3s_common.h"
+
+// Device scratch of f3s_preprocess_count_static, owned by the library instead of the caller: every
+// GPU the library runs on holds its own copy (8 MiB) at its own address until the process ends.
+// In host code the name below is only a handle for hipGetSymbolAddress, never an address.
+static constexpr size_t kF3sStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kF3sStaticScratchBytes];
 
 namespace f3s {
 namespace {
@@ -782,19 +790,16 @@ size_t preprocess_workspace_bytes(int N, int /*E*/) {
   return kWsHeaderBytes + 3 * align256(nRW * sizeof(int32_t));
 }
 
-int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
-                            int W, int32_t* blockPartition, int32_t* edgeToColumn,
-                            int32_t* edgeToRow, int32_t* rowWindowOffset,
-                            int32_t* sortedRowWindows, void* workspace, size_t wsBytes,
-                            int64_t* nTcbHost, hipStream_t stream) {
-  if (H != 16 || (W != 16 && W != 8))
-    return fail(-2, "f3s_preprocess_count: block %dx%d unsupported (16x16 or 16x8)", H, W);
-  if (N < 0 || E < 0) return fail(-2, "f3s_preprocess_count: negative size");
-  if (wsBytes < preprocess_workspace_bytes(N, E))
-    return fail(-2, "f3s_preprocess_count: workspace %zu B < required %zu B", wsBytes,
-                preprocess_workspace_bytes(N, E));
+namespace {
+
+// Enqueues every kernel of phase 1 on `stream`; `ws` is device scratch of
+// preprocess_workspace_bytes(N, E) bytes whose header ends up holding the TC-block total and the
+// error flag.
+int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int W,
+                  int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                  int32_t* rowWindowOffset, int32_t* sortedRowWindows, char* ws,
+                  hipStream_t stream) {
   const int nRW = (N + kWinRows - 1) / kWinRows;
-  char* ws = static_cast<char*>(workspace);
   WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
   const size_t seg = align256((size_t)nRW * sizeof(int32_t));
   int32_t* keysA = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes);
@@ -852,11 +857,96 @@ int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N,
   hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
                      nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
   F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+int check_count_args(const char* who, int N, int E, int H, int W) {
+  if (H != 16 || (W != 16 && W != 8))
+    return fail(-2, "%s: block %dx%d unsupported (16x16 or 16x8)", who, H, W);
+  if (N < 0 || E < 0) return fail(-2, "%s: negative size", who);
+  return 0;
+}
+
+}  // namespace
+
+int launch_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                            int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                            int32_t* edgeToRow, int32_t* rowWindowOffset,
+                            int32_t* sortedRowWindows, void* workspace, size_t wsBytes,
+                            int64_t* nTcbHost, hipStream_t stream) {
+  if (int rc = check_count_args("f3s_preprocess_count", N, E, H, W)) return rc;
+  if (wsBytes < preprocess_workspace_bytes(N, E))
+    return fail(-2, "f3s_preprocess_count: workspace %zu B < required %zu B", wsBytes,
+                preprocess_workspace_bytes(N, E));
+  char* ws = static_cast<char*>(workspace);
+  if (int rc = enqueue_count(rowPtr, colIdx, N, E, W, blockPartition, edgeToColumn, edgeToRow,
+                             rowWindowOffset, sortedRowWindows, ws, stream))
+    return rc;
   WsHeader host;
-  F3S_HIP_CHECK(hipMemcpyAsync(&host, hdr, sizeof(WsHeader), hipMemcpyDeviceToHost, stream));
+  F3S_HIP_CHECK(hipMemcpyAsync(&host, ws, sizeof(WsHeader), hipMemcpyDeviceToHost, stream));
   F3S_HIP_CHECK(hipStreamSynchronize(stream));
   if (host.error) return fail(-4, "f3s_preprocess_count: column index outside [0, %d)", N);
   *nTcbHost = host.nTcb;
+  return 0;
+}
+
+// ------------------------------------------------------- phase 1 without any allocation
+// The scratch is the file-scope array `scratch` at the top of this file; host code reaches it
+// through the per-device address hipGetSymbolAddress returns, looked up once per device.
+constexpr size_t kStaticScratchBytes = kF3sStaticScratchBytes;
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMutex;
+void* g_scratchPtr[kMaxDevices] = {};
+
+int static_scratch(char** out) {
+  int dev = -1;
+  F3S_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(-2, "f3s_preprocess_count_static: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratchMutex);
+  if (!g_scratchPtr[dev]) {
+    void* ptr = nullptr;
+    F3S_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_scratchPtr[dev] = ptr;
+  }
+  *out = static_cast<char*>(g_scratchPtr[dev]);
+  return 0;
+}
+
+__global__ void publish_result_kernel(const WsHeader* __restrict__ hdr,
+                                      long long* __restrict__ result) {
+  result[0] = hdr->nTcb;
+  result[1] = (long long)hdr->error;
+}
+
+}  // namespace
+
+size_t preprocess_static_scratch_bytes() { return kStaticScratchBytes; }
+
+int launch_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, int N, int E,
+                                   int H, int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                                   int32_t* edgeToRow, int32_t* rowWindowOffset,
+                                   int32_t* sortedRowWindows, int64_t* resultDev,
+                                   hipStream_t stream) {
+  if (int rc = check_count_args("f3s_preprocess_count_static", N, E, H, W)) return rc;
+  if (preprocess_workspace_bytes(N, E) > kStaticScratchBytes)
+    return fail(-5, "f3s_preprocess_count_static: a graph of %d nodes needs %zu B of scratch, the "
+                    "library's own buffer holds %zu B; use f3s_preprocess_count with a workspace",
+                N, preprocess_workspace_bytes(N, E), kStaticScratchBytes);
+  char* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // every kernel below starts from a header it clears itself and overwrites whatever else it
+  // reads of the buffer, so nothing of an earlier call survives into this one
+  if (int rc = enqueue_count(rowPtr, colIdx, N, E, W, blockPartition, edgeToColumn, edgeToRow,
+                             rowWindowOffset, sortedRowWindows, ws, stream))
+    return rc;
+  hipLaunchKernelGGL(publish_result_kernel, dim3(1), dim3(1), 0, stream,
+                     reinterpret_cast<const WsHeader*>(ws),
+                     reinterpret_cast<long long*>(resultDev));
+  F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
 

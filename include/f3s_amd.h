@@ -64,6 +64,28 @@ int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, in
                          size_t ws_bytes, int64_t* nTCB_host, void* stream);
 
 /*
+ * f3s_preprocess_count for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+ * inputs and outputs as f3s_preprocess_count, with two differences:
+ *   - the scratch is a buffer the library owns, a static device array of
+ *     f3s_preprocess_static_scratch_bytes() = 8 MiB per GPU that lives until the process ends;
+ *     graphs needing more (f3s_preprocess_workspace_bytes(N, E) > 8 MiB, i.e. above about
+ *     11.1 million nodes) are rejected with status -5 and a message;
+ *   - nothing is copied to the host and the stream is not synchronised: result_dev is a DEVICE
+ *     pointer to two int64, out: {total TC blocks, 1 if a column index lay outside [0, N) else 0}.
+ * The call makes no hipMalloc / hipFree and uses no allocating library routine; everything is
+ * enqueued on `stream` (kernels only, no memset nodes). Every call on a GPU shares that GPU's
+ * buffer: calls that overlap on one GPU (different streams, different threads) race; calls that
+ * follow each other on one stream, or are otherwise ordered, are safe, and each call clears what
+ * it needs cleared.
+ */
+size_t f3s_preprocess_static_scratch_bytes(void);
+int f3s_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                                int W, int32_t* blockPartition, int32_t* edgeToColumn,
+                                int32_t* edgeToRow, int32_t* rowWindowOffset,
+                                int32_t* sortedRowWindows, int64_t* result_dev, void* stream);
+
+/*
  * Phase 2 of F3S.preprocess_gpu: the outputs sized by nTCB. Replaces
  * generate_tcblock_rowid_cuda (src/utils.cu:53-78), generate_tcoffset_id_atob_cuda with
  * update_bitmap (src/utils.cu:23-36, 173-267) and the inclusive scan into tcblock_offset
