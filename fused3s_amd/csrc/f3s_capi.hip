@@ -110,8 +110,9 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
     return f3s::fail(-1, "f3s_attention_fwd: null pointer");
   if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
       f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
-      f3s::misaligned(tcbBitMap, 8))
-    return f3s::fail(-1, "f3s_attention_fwd: Q/K/V/out/sparseAToXidx need 16-byte alignment");
+      f3s::misaligned(tcbBitMap, 16))
+    return f3s::fail(-1, "f3s_attention_fwd: Q/K/V/out/sparseAToXidx/tcbBitMap need 16-byte "
+                         "alignment");
   if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd: negative nTCB");
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd: null TC-block arrays");
@@ -133,8 +134,9 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
     return f3s::fail(-1, "f3s_attention_fwd_heads: null pointer");
   if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
       f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
-      f3s::misaligned(tcbBitMap, 8))
-    return f3s::fail(-1, "f3s_attention_fwd_heads: Q/K/V/out/sparseAToXidx need 16-byte alignment");
+      f3s::misaligned(tcbBitMap, 16))
+    return f3s::fail(-1, "f3s_attention_fwd_heads: Q/K/V/out/sparseAToXidx/tcbBitMap need "
+                         "16-byte alignment");
   if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd_heads: negative nTCB");
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd_heads: null TC-block arrays");
@@ -152,14 +154,15 @@ int f3s_attention_fwd_tcb8(const int32_t* rowWindowOffset, const int32_t* window
   if (!rowWindowOffset || !Q || !K || !V || !out)
     return f3s::fail(-1, "f3s_attention_fwd_tcb8: null pointer");
   if (f3s::misaligned(Q, 16) || f3s::misaligned(K, 16) || f3s::misaligned(V, 16) ||
-      f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 4) ||
-      f3s::misaligned(tcbBitMap, 8) || f3s::misaligned(sddmmResult, 16))
-    return f3s::fail(-1, "f3s_attention_fwd_tcb8: Q/K/V/out/sddmmResult need 16-byte alignment");
+      f3s::misaligned(out, 16) || f3s::misaligned(sparseAToXidx, 16) ||
+      f3s::misaligned(tcbBitMap, 16) || f3s::misaligned(sddmmResult, 16))
+    return f3s::fail(-1, "f3s_attention_fwd_tcb8: Q/K/V/out/sparseAToXidx/tcbBitMap/sddmmResult "
+                         "need 16-byte alignment");
   if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd_tcb8: negative nTCB");
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd_tcb8: null TC-block arrays");
   return f3s::launch_attention_tcb8(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, d,
-                                    Q, K, V, applySoftmax, out, sddmmResult,
+                                    Q, K, V, applySoftmax, out, sddmmResult, nTCB,
                                     static_cast<hipStream_t>(stream));
 }
 

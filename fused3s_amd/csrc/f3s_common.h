@@ -37,7 +37,7 @@ int launch_attention_heads(const int32_t* rowWindowOffset, const int32_t* window
 int launch_attention_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                           const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
                           const void* Q, const void* K, const void* V, int applySoftmax,
-                          float* out, float* sddmm, hipStream_t stream);
+                          float* out, float* sddmm, int64_t nTcb8, hipStream_t stream);
 
 int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype);
 
@@ -47,14 +47,14 @@ int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windo
                             const int32_t* sparseAToXidx, const uint64_t* bitmap, int N, int d,
                             int dtype, const void* Q, const void* K, const void* V,
                             float scaleLog2, int applySoftmax, float* out, void* workspace,
-                            size_t wsBytes, hipStream_t stream);
+                            size_t wsBytes, int64_t nTcb, hipStream_t stream);
 
 int launch_attention_short_windows(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                                    const int32_t* sparseAToXidx, const uint64_t* bitmap, int N,
                                    int d, int dtype, const void* Q, const void* K, const void* V,
                                    float scaleLog2, int applySoftmax, float* out, int nHeads,
                                    int ldIn, int ldOut, int maxBlocks, int longPrefix,
-                                   hipStream_t stream);
+                                   int64_t nTcb, hipStream_t stream);
 
 // preprocessing (f3s_preprocess.hip)
 size_t preprocess_workspace_bytes(int N, int E);

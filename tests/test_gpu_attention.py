@@ -172,7 +172,7 @@ def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
                                       pre["tcbBitMap"], N, Q, K, V, 1.0, applySoftmax=False)
     got_n = gpu_attention(pre, N, Q, K, V, 1.0, pre["sortedRowWindows"], softmax=False, sliced=True)
     assert np.abs(got_n - want_n).max() < 2e-2 * max(1.0, np.abs(want_n).max())
-    # bf16 inputs through the same schedule (P rounded to bf16: mean-relative bar 4e-3)
+    # bf16 inputs through the same schedule, same bar
     as_bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
     Qb, Kb, Vb = (torch.as_tensor(x.astype(np.float32)).to(torch.bfloat16) for x in (Q, K, V))
     want_b = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
@@ -188,7 +188,7 @@ def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
     got_b = capi.attention(rwo, od, atox, bm, N, Qb.to(dev), Kb.to(dev), Vb.to(dev), scale,
                            workspace=ws).cpu().numpy()
     assert np.abs(got_b - want_b).max() < MAX_ABS
-    assert mean_rel(got_b, want_b) < 4e-3
+    assert mean_rel(got_b, want_b) < 1e-3
 
 
 @pytest.mark.parametrize("d", [32, 64, 128])

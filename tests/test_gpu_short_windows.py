@@ -10,7 +10,7 @@ from conftest import random_csr
 
 pytestmark = pytest.mark.gpu
 MAX_ABS = 2e-2
-MEAN_REL = {torch.float16: 1e-3, torch.bfloat16: 4e-3}
+MEAN_REL = {torch.float16: 1e-3, torch.bfloat16: 1e-3}
 
 
 def bits(t):
