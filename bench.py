@@ -2,11 +2,14 @@
 """Benchmark of the fused 3S attention hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3_chunglu_233k]
+                    [--no-other-configs] [--no-cpu-baseline]
 
 A step is one launch of the fused SDDMM -> softmax -> SpMM kernel (through the C ABI,
 f3s_attention_fwd, heavy-first window order) over the whole synthetic graph, with the CSR,
 the TC-block structure and Q/K/V already resident in HBM. Preprocessing is timed separately and
-reported in the same JSON line. Prints exactly one JSON line on stdout; progress goes to stderr.
+reported in the same JSON line, as are compact results of the other benchmark configurations
+(`other_configs`) and a sanity check of the timed output. Prints exactly one JSON line on stdout;
+progress goes to stderr.
 
 Figures (all exact functions of the generated graph):
   value              effective TFLOP/s  = 4*d*E / t                    (useful flops over edges)
@@ -111,57 +114,39 @@ def cpu_baseline_torch(rowPtr, colIdx, N, Q, K, V, scale, d, max_edges=4_000_000
                       "%d rows (%d edges), %.2f s" % (rows_n, e, dt)}
 
 
-def measured_traffic(args, sliced):
-    """HBM-side bytes per attention call from rocprofv3 (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000,
-    factors from a 1 GiB copy; profiles/f3s_fwd_kernel_d64_cfg3_chunglu_233k.md). Counters cannot
-    be read from inside this process, so the figure is the recorded one and is only given for the
-    workload and schedule it was measured on."""
-    if args.config == "cfg3_chunglu_233k" and args.scale == 1.0 and not args.natural_order:
-        if sliced:
-            # slice_index_kernel + f3s_fwd_unit_kernel + f3s_merge_slices_kernel
-            return (2 * (42_397 + 2_642_050 + 262_572) + 512 + 524_196 + 58_270) * 1024
-        return (2 * 7_353_770 + 58_241) * 1024
+def recorded_traffic(config, schedule, scale, natural_order):
+    """HBM-side bytes per attention call as rocprofv3 counted them in an EARLIER run (FETCH_SIZE
+    and WRITE_SIZE, scaled by what the same counters read for a plain copy): counters cannot be
+    read from inside this process, so the figure is a record, labelled with the profile summary
+    it comes from, and is only given for the workload and schedule it was taken on."""
+    path = os.path.join(ROOT, "profiles", "traffic_recorded.json")
+    if scale != 1.0 or natural_order or not os.path.exists(path):
+        return None
+    for rec in json.load(open(path)).get("records", []):
+        if rec.get("config") == config and rec.get("schedule") == schedule:
+            return rec
     return None
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="cfg3_chunglu_233k")
-    ap.add_argument("--scale", type=float, default=1.0, help="shrink the graph (debugging)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
-    ap.add_argument("--cpu-budget", type=float, default=12.0)
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
-                         "FETCH_SIZE / WRITE_SIZE counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        log("bench.py: this build runs on ONE GPU (row windows would shard across GPUs with K/V "
-            "replicated, but no multi-GPU path is part of it); run with --gpus 1")
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        log("bench.py: no GPU visible; the HIP path has no CPU fallback")
-        sys.exit(3)
-
+def run_config(name, args, dev, headline):
+    """Generate one configuration, preprocess it, time the attention call; returns the result
+    dict (the full line for the headline configuration, a compact one otherwise)."""
     from fused3s_amd import capi, synth
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    cfg = synth.CONFIGS[args.config]
+    cfg = synth.CONFIGS[name]
     d = cfg["d"]
     heads = cfg["heads"]
     tdtype = torch.float16 if cfg["dtype"] == "fp16" else torch.bfloat16
+    scale_graph = args.scale if headline else 1.0
 
     t0 = time.time()
-    rowPtr, colIdx = synth.make_graph(args.config, seed=0, device=dev, scale=args.scale)
+    rowPtr, colIdx = synth.make_graph(name, seed=0, device=dev, scale=scale_graph)
     torch.cuda.synchronize()
     N = rowPtr.numel() - 1
     E = colIdx.numel()
     deg = (rowPtr[1:] - rowPtr[:-1])
+    max_degree = int(deg.max())
     log("graph %s: N=%d E=%d max_degree=%d (%.1f s to generate on the GPU)"
-        % (args.config, N, E, int(deg.max()), time.time() - t0))
+        % (name, N, E, max_degree, time.time() - t0))
     # single head: [N, d] ~ N(0, 1); multi-head: [N, heads, d] ~ N(0, 1/d)
     Q, K, V = synth.features(N, heads * d, seed=0, device=dev, dtype=tdtype,
                              std=1.0 if heads == 1 else d ** -0.5)
@@ -182,10 +167,14 @@ def main():
     nTCB = pre["blockCount"]
     nRW = (N + 15) // 16
     cnt = (pre["rowWindowOffset"][1:] - pre["rowWindowOffset"][:-1])
-    log("preprocess: nTCB=%d nRW=%d max TCB/window=%d mean=%.1f  %.2f ms (%.2f G edges/s)"
-        % (nTCB, nRW, int(cnt.max()), float(cnt.float().mean()), pre_ms, E / pre_ms / 1e6))
+    # scan bound of the preprocessing: CSR read once, ids + bitmaps written once
+    pre_bytes = 4.0 * E + 4.0 * (N + 1) + 96.0 * nTCB
+    pre_hbm_frac = pre_bytes / (pre_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS
+    log("preprocess: nTCB=%d nRW=%d max TCB/window=%d mean=%.1f  %.2f ms (%.2f G edges/s, %.1f%% "
+        "of the HBM scan bound)" % (nTCB, nRW, int(cnt.max()), float(cnt.float().mean()), pre_ms,
+                                    E / pre_ms / 1e6, 100 * pre_hbm_frac))
 
-    if args.calibrate_copy:
+    if headline and args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
         dst = torch.empty_like(src)
         for _ in range(3):
@@ -193,37 +182,52 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    order = None if args.natural_order else pre["sortedRowWindows"]
+    natural = headline and args.natural_order
+    order = None if natural else pre["sortedRowWindows"]
     out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
     # scratch of the column-sliced schedule, which the library picks for graphs with long windows
-    workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype)
+    workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype) if heads == 1 else None
+    schedule = "column-sliced" if workspace is not None else "window"
     log("attention schedule: %s" % ("column-sliced (%.0f MB workspace)" % (workspace.numel() / 1e6)
                                     if workspace is not None else "workgroup per window"))
 
     if heads == 1:
-        def step():
+        def step(v=V, o=out):
             capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"], pre["tcbBitMap"],
-                           N, Q, K, V, scale, True, out=out, workspace=workspace)
+                           N, Q, K, v, scale, True, out=o, workspace=workspace)
     else:
-        def step():
+        def step(v=V, o=out):
             capi.attention_heads(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
-                                 pre["tcbBitMap"], N, Q, K, V, scale, True, out=out)
+                                 pre["tcbBitMap"], N, Q, K, v, scale, True, out=o)
 
-    for _ in range(args.warmup):
+    steps, warmup = (args.steps, args.warmup) if headline else (10, 3)
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
     events[0].record()
-    for i in range(args.steps):
+    for i in range(steps):
         step()
         events[i + 1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    kern_ms = np.array([events[i].elapsed_time(events[i + 1]) for i in range(args.steps)])
-    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = np.array([events[i].elapsed_time(events[i + 1]) for i in range(steps)])
+    ms_per_step = wall * 1e3 / steps
     t_avg = float(kern_ms.mean()) * 1e-3
     t_med = float(np.median(kern_ms)) * 1e-3
+
+    # sanity of what was timed: finite output, and softmax weights that sum to one (with V = 1
+    # every row that has an edge must come out as 1, every other row as 0)
+    finite = bool(torch.isfinite(out).all())
+    ones = torch.ones_like(V)
+    o1 = torch.empty_like(out)
+    step(ones, o1)
+    torch.cuda.synchronize()
+    has = (deg > 0).unsqueeze(1).to(o1.dtype)
+    rowsum_err = float((o1 - has).abs().max())
+    del ones, o1
+    sanity = {"finite": finite, "rowsum_max_err": rowsum_err, "ok": finite and rowsum_err < 2e-3}
 
     D = heads * d  # all per-node byte and flop counts scale with the concatenated width
     f_eff = 4.0 * D * E
@@ -234,41 +238,53 @@ def main():
     achieved = f_mfma / t_avg / 1e12
 
     # the bound that binds on paper: t_roof = max(F_mfma / P_mfma, B_min / BW_hbm)
-    traffic = measured_traffic(args, workspace is not None)
     if f_mfma / (PEAK_MFMA_F16_TFLOPS * 1e12) >= b_min / (PEAK_HBM_GBPS * 1e9):
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": traffic}
+                    "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": None}
     else:
         gbps = b_min / t_avg / 1e9
         roofline = {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic}
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": None}
+    log("%s kernel: median %.3f ms  mean %.3f ms  effective %.1f TFLOP/s  MFMA %.1f TFLOP/s "
+        "(%.1f%%)  gather %.0f GB/s  sanity %s"
+        % (name, t_med * 1e3, t_avg * 1e3, f_eff / t_med / 1e12, achieved,
+           100 * achieved / PEAK_MFMA_F16_TFLOPS, b_gather / t_med / 1e9, sanity))
+    if not headline:
+        return {"config": name, "N": N, "E": E, "nTCB": nTCB, "d": d, "heads": heads,
+                "dtype": "f16" if cfg["dtype"] == "fp16" else "bf16", "schedule": schedule,
+                "kernel_ms_median": t_med * 1e3, "effective_tflops": f_eff / t_med / 1e12,
+                "bound": roofline["bound"], "achieved": roofline["achieved"],
+                "frac": roofline["frac"], "gather_gbps": b_gather / t_med / 1e9,
+                "preprocess_ms": pre_ms, "preprocess_hbm_frac": pre_hbm_frac,
+                "sanity_ok": sanity["ok"]}
+
     result = {
         "metric": "fused_3s_attention_effective_tflops_d%d_%s%s"
                   % (d, cfg["dtype"], "" if heads == 1 else "_%dheads" % heads),
-        "value": f_eff / (wall / args.steps) / 1e12,
+        "value": f_eff / (wall / steps) / 1e12,
         "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if cfg["dtype"] == "fp16" else "bf16", "data": "synthetic",
         "config": {"workload": "%s: N=%d E=%d d=%d %s %s, scalingFactor=sqrt(d), %s window order"
-                               % (args.config, N, E, d, cfg["dtype"],
+                               % (name, N, E, d, cfg["dtype"],
                                   "single head" if heads == 1 else
                                   "%d heads in one launch, output [N, %d]" % (heads, D),
-                                  "natural" if args.natural_order else "heavy-first"),
+                                  "natural" if natural else "heavy-first"),
                    "nTCB": nTCB, "nRW": nRW, "max_tcb_per_window": int(cnt.max()),
-                   "scale": args.scale},
+                   "max_degree": max_degree, "scale": scale_graph},
         "kernel_ms_median": t_med * 1e3, "kernel_ms_mean": t_avg * 1e3,
         "padded_tflops": f_pad / t_med / 1e12,
         "hbm_min_gbps": b_min / t_med / 1e9, "hbm_min_frac": b_min / t_med / 1e9 / PEAK_HBM_GBPS,
         "gather_gbps": b_gather / t_med / 1e9,
         "preprocess_ms": pre_ms, "preprocess_gedges_per_s": E / pre_ms / 1e6,
-        "schedule": "column-sliced" if workspace is not None else "window",
+        "preprocess_hbm_frac": pre_hbm_frac,
+        "schedule": schedule,
+        "sanity": sanity,
         "roofline": roofline,
+        "traffic_recorded": recorded_traffic(name, schedule, scale_graph, natural),
     }
-    log("kernel: median %.3f ms  mean %.3f ms  effective %.1f TFLOP/s  MFMA %.1f TFLOP/s (%.1f%%)"
-        % (t_med * 1e3, t_avg * 1e3, f_eff / t_med / 1e12, achieved,
-           100 * achieved / PEAK_MFMA_F16_TFLOPS))
     if heads > 1:
         # the reference's way: one launch per head on contiguous per-head copies
         per_head = [tuple(x[:, h].contiguous() for x in (Q, K, V)) for h in range(heads)]
@@ -280,14 +296,14 @@ def main():
                                pre["tcbBitMap"], N, *per_head[h], scale, True, out=outs[h])
         loop()
         torch.cuda.synchronize()
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         ev[0].record()
-        for i in range(args.steps):
+        for i in range(steps):
             loop()
             ev[i + 1].record()
         torch.cuda.synchronize()
         result["per_head_loop_ms_median"] = float(np.median(
-            [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]))
+            [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]))
         log("per-head loop of %d single-head launches: median %.3f ms"
             % (heads, result["per_head_loop_ms_median"]))
     if not args.no_cpu_baseline:
@@ -300,6 +316,47 @@ def main():
         log("cpu baseline (PyTorch ops):", result["cpu_baseline_torch"])
     else:
         result["cpu_baseline"] = None
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg3_chunglu_233k")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the graph (debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the compact lines of the other benchmark configurations")
+    ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
+    ap.add_argument("--cpu-budget", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU (row windows would shard across GPUs with K/V "
+            "replicated, but no multi-GPU path is part of it); run with --gpus 1")
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the HIP path has no CPU fallback")
+        sys.exit(3)
+
+    from fused3s_amd import synth
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    result = run_config(args.config, args, dev, headline=True)
+    if not args.no_other_configs:
+        # the other benchmark configurations, one compact entry each (kernel time, the bound that
+        # binds on paper and the fraction reached, preprocessing time)
+        others = []
+        for name in synth.CONFIGS:
+            if name == args.config:
+                continue
+            torch.cuda.empty_cache()
+            others.append(run_config(name, args, dev, headline=False))
+        result["other_configs"] = others
     print(json.dumps(result), flush=True)
 
 

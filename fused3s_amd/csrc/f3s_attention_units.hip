@@ -272,7 +272,11 @@ int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* ato
                      stream, rwo, atox, nRW, S, sliceWidth, sliceStart);
   F3S_HIP_CHECK(hipGetLastError());
   const int nGroups = (nRW + kUnitWaves - 1) / kUnitWaves;
+#ifdef F3S_PROBE_LDS_PAD
+  constexpr size_t lds = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES + F3S_PROBE_LDS_PAD;
+#else
   constexpr size_t lds = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES;
+#endif
   if (int rc = allow_lds(f3s_fwd_unit_kernel<ET, D, SOFTMAX, true, false>, lds)) return rc;
   hipLaunchKernelGGL((f3s_fwd_unit_kernel<ET, D, SOFTMAX, true, false>),
                      dim3((unsigned)(P * nGroups * kXcds)), dim3(kUnitWaves * 64), lds, stream,

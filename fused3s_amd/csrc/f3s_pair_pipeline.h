@@ -54,6 +54,23 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 
 #define F3S_LDS __attribute__((address_space(3)))
 
+// probe builds can drop one part of a step (results are then wrong on purpose)
+#ifdef F3S_PROBE_NO_READ
+#define F3S_ABL_READ(x) op = Operands{}
+#else
+#define F3S_ABL_READ(x) x
+#endif
+#ifdef F3S_PROBE_NO_GATHER
+#define F3S_ABL_GATHER(x) (void)0
+#else
+#define F3S_ABL_GATHER(x) x
+#endif
+#ifdef F3S_PROBE_NO_COMPUTE
+#define F3S_ABL_COMPUTE(x) consume(op)
+#else
+#define F3S_ABL_COMPUTE(x) x
+#endif
+
 template <typename ET, int L>
 struct Vec {
   typedef ET type __attribute__((ext_vector_type(L)));
@@ -348,6 +365,9 @@ struct PairPipeline {
 #pragma unroll
     for (int i = 0; i < T; i++) {
       pin(rows[i]);
+#ifdef F3S_PROBE_ROWMASK
+      rows[i] &= F3S_PROBE_ROWMASK;
+#endif
       const uint32_t ro = HEADS ? __umul24((uint32_t)rows[i], rowBytes)
                                 : (uint32_t)rows[i] * (uint32_t)G::ROW;
       const uint32_t ko = ro + gatherOffK[i];
@@ -389,6 +409,19 @@ struct PairPipeline {
   // LDS distance between the rows of slot s and slot s + 16 of a tile
   static __device__ __forceinline__ constexpr int v_half_distance() {
     return (lds_row_of<D>(16) - lds_row_of<D>(0)) * G::ROW;
+  }
+
+  __device__ __forceinline__ void consume(Operands& op) {
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int i = 0; i < KS; i++) pin(op.k[b][i]);
+#pragma unroll
+    for (int j = 0; j < T; j++) {
+      pin(op.v[j][0]);
+      pin(op.v[j][1]);
+    }
+    pin(op.words);
   }
 
   // nValid: blocks of the structure that exist in this step (1..BPS); only the last step of a
@@ -552,19 +585,19 @@ struct PairPipeline {
       vm_wait<0>();                                                                            \
     }                                                                                          \
     Operands op;                                                                               \
-    read_operands<STAGE_IDX, Q4>((p >> 2) & 1, op);                                            \
+    F3S_ABL_READ((read_operands<STAGE_IDX, Q4>((p >> 2) & 1, op)));                            \
     lds_wait();                                                                                \
     __builtin_amdgcn_sched_barrier(0);                                                         \
     if constexpr (Q4 == 0) {                                                                   \
       metaIssued = (p >> 2) + 1 <= (nSteps - 1) >> 2;                                          \
       if (metaIssued) issue_meta(pb, t0, t1, (p >> 2) + 1);                                    \
     }                                                                                          \
-    if (more) issue_gather<STAGE_IDX, GQ4>(pb, ((p + NS) >> 2) & 1);                           \
+    if (more) F3S_ABL_GATHER((issue_gather<STAGE_IDX, GQ4>(pb, ((p + NS) >> 2) & 1)));         \
     __builtin_amdgcn_sched_barrier(0);                                                         \
     {                                                                                          \
       const int tFirst = t0 + p * BPS;                                                         \
       const int left = t1 - tFirst;                                                            \
-      compute(pb, op, tFirst, left < BPS ? left : BPS);                                        \
+      F3S_ABL_COMPUTE(compute(pb, op, tFirst, left < BPS ? left : BPS));                       \
     }                                                                                          \
     p++;                                                                                       \
     if (p >= nSteps) break;                                                                    \
