@@ -27,6 +27,8 @@
 //                        in CSR order (src/utils.cu:173-224, 23-36, 53-65).
 //
 // All results are bit-identical to the reference's algorithm with edgeToRow[e] = row(e).
+#include <hipcub/hipcub.hpp>
+
 #include <mutex>
 
 #include "f3s_common.h"
@@ -43,8 +45,12 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kRangeMax = 393216;  // columns per bitset pass: 48 KiB of bits + 12 KiB of prefixes
 constexpr int kSortMax = 1024;     // windows up to this many edges are ranked by a per-wave LDS sort
-constexpr int kFillChunk = 512;    // TC blocks held in LDS at once by window_fill_kernel
-constexpr int kFillChunkSmall = 128;  // the same for graphs of short windows (one wave each)
+// TC blocks held in LDS at once by window_fill_kernel: windows with strictly ascending rows (96
+// bytes of LDS per 16x16 block) and windows with repeated or descending columns (96 bytes as
+// well, but a second pass per chunk)
+constexpr int kFillChunk = 640;
+constexpr int kFillChunkGeneric = 512;
+constexpr int kFillChunkSmall = 128;  // both, for graphs of short windows (one wave each)
 
 // workspace header (bytes 0..255): int64 nTCB, int32 error flag, and the queue of windows too
 // long for the wave-per-window kernel (filled by window_rank_small_kernel, drained by
@@ -54,6 +60,8 @@ struct WsHeader {
   int error;
   int nBig;     // entries in the queue
   int nextBig;  // next entry to hand out
+  int maxCount; // largest per-window block count (multi-workgroup finalize)
+  int nextMed;  // next queue entry to hand out to window_rank_sort_kernel
 };
 constexpr size_t kWsHeaderBytes = 256;
 
@@ -316,7 +324,7 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
     int nPasses, int32_t* __restrict__ blockPartition,
     int32_t* __restrict__ edgeToColumn,
     int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
-    const int32_t* __restrict__ bigList) {
+    const int32_t* __restrict__ bigList, int skipUpTo) {
   extern __shared__ __align__(16) uint32_t smem[];
   uint32_t* bits = smem;                 // range/32 words
   uint32_t* pref = smem + (range >> 5);  // range/128 group prefixes
@@ -344,6 +352,7 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
   __syncthreads();
   const int eS = sRow[0], eE = sRow[16];
   if (!bigList && eE - eS <= kSortMax) break;  // ranked by window_rank_small_kernel
+  if (bigList && eE - eS <= skipUpTo) continue;  // ranked by window_rank_sort_kernel
   const int nGroups = range >> 7;
   unsigned uniqueBefore = 0;
   for (int pass = 0; pass < nPasses; pass++) {
@@ -422,6 +431,115 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
   for (int e = eS + tid; e < eE; e += TB) edgeToRow[e] = r0 + row_of_edge(sRow, e);
   if (tid == 0) blockPartition[w] = (int)((uniqueBefore + W - 1) / W);
   if (!bigList) break;
+  }
+}
+
+// Windows of kSortMax < edges <= kMedMax on graphs whose column range needs several bitset passes
+// (N > kRangeMax): one workgroup per queued window sorts the window's column ids (block-wide
+// radix sort), compacts the distinct ones and ranks every edge by binary search, instead of
+// several passes over a 48 KiB bitset that such a window fills with a few thousand bits.
+constexpr int kMedThreads = 256;
+constexpr int kMedItems = 16;
+constexpr int kMedMax = kMedThreads * kMedItems;
+
+template <int W>
+__global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int colBits,
+    int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
+    const int32_t* __restrict__ bigList) {
+  typedef hipcub::BlockRadixSort<unsigned, kMedThreads, kMedItems> Sort;
+  __shared__ union {
+    typename Sort::TempStorage sort;
+    unsigned keys[kMedMax];
+  } u;
+  __shared__ unsigned sUniq[kMedMax];
+  __shared__ int sRow[17];
+  __shared__ unsigned sWaveTot[kMedThreads / 64];
+  __shared__ int sTake;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int nBig = hdr->nBig;
+  while (true) {
+    __syncthreads();
+    if (tid == 0) sTake = atomicAdd(&hdr->nextMed, 1);
+    __syncthreads();
+    if (sTake >= nBig) break;
+    const int w = bigList[sTake];
+    const int r0 = w * 16;
+    if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
+    __syncthreads();
+    const int eS = sRow[0], eE = sRow[16];
+    const int n = eE - eS;
+    if (n > kMedMax) continue;  // left to window_rank_kernel
+    unsigned keys[kMedItems];
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < kMedItems; j++) {
+      const int i = tid * kMedItems + j;
+      unsigned k = 0xFFFFFFFFu;  // padding sorts last
+      if (i < n) {
+        k = (unsigned)colIdx[eS + i];
+        if (k >= (unsigned)N) {
+          bad = true;
+          k = 0u;
+        }
+      }
+      keys[j] = k;
+    }
+    if (bad) atomicOr(&hdr->error, 1);
+    // one bit above the column ids keeps the padding behind every real key
+    Sort(u.sort).Sort(keys, 0, colBits + 1 < 32 ? colBits + 1 : 32);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMedItems; j++) u.keys[tid * kMedItems + j] = keys[j];
+    __syncthreads();
+    // distinct columns: first occurrences, compacted in order
+    unsigned cnt = 0;
+    unsigned firstMask = 0;
+#pragma unroll
+    for (int j = 0; j < kMedItems; j++) {
+      const int i = tid * kMedItems + j;
+      const bool first = i < n && (i == 0 || u.keys[i - 1] != keys[j]);
+      firstMask |= first ? (1u << j) : 0u;
+      cnt += first ? 1u : 0u;
+    }
+    const unsigned incl = wave_inclusive_scan(cnt, lane);
+    if (lane == 63) sWaveTot[wave] = incl;
+    __syncthreads();
+    unsigned waveOff = 0, nUniq = 0;
+#pragma unroll
+    for (int v = 0; v < kMedThreads / 64; v++) {
+      const unsigned x = sWaveTot[v];
+      if (v < wave) waveOff += x;
+      nUniq += x;
+    }
+    unsigned pos = waveOff + incl - cnt;
+#pragma unroll
+    for (int j = 0; j < kMedItems; j++)
+      if ((firstMask >> j) & 1u) sUniq[pos++] = keys[j];
+    __syncthreads();
+    for (int e = eS + tid; e < eE; e += kMedThreads) {
+      unsigned col = (unsigned)colIdx[e];
+      if (col >= (unsigned)N) col = 0u;
+      int lo = 0, hi = (int)nUniq - 1, found = 0;
+      while (lo <= hi) {
+        const int mid = (lo + hi) >> 1;
+        const unsigned v = sUniq[mid];
+        if (v == col) {
+          found = mid;
+          break;
+        }
+        if (v < col)
+          lo = mid + 1;
+        else
+          hi = mid - 1;
+      }
+      edgeToColumn[e] = found;
+      edgeToRow[e] = r0 + row_of_edge(sRow, e);
+    }
+    if (tid == 0) blockPartition[w] = (int)((nUniq + W - 1) / W);
   }
 }
 
@@ -568,35 +686,231 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   }
 }
 
+// ---- the same scan + stable sort spread over many workgroups, for graphs with many windows.
+// Every WAVE of the grid owns a contiguous chunk of the windows (chunks in wave order), exactly as
+// the waves of finalize_count_kernel do; what that kernel exchanges through LDS and block barriers
+// goes through small global arrays and kernel boundaries here:
+//   finalize_partials_kernel   per-wave sum and maximum of the block counts
+//   finalize_scan_kernel       rowWindowOffset of the chunk (carry = sums of the earlier waves),
+//                              total and maximum into the header, digit histogram of pass 0
+//   finalize_scatter_kernel    one pass: start of (digit, wave) from every wave's histogram, then
+//                              the in-order scatter of the chunk
+//   finalize_histogram_kernel  digit histogram of the next pass (its input is the scattered
+//                              order, complete only at the kernel boundary)
+// The number of passes depends on the largest count, known on the device only: the host enqueues
+// as many passes as the window count could need and the surplus kernels return at once.
+constexpr int kFinDigitBits = 6;
+constexpr int kFinBins = 1 << kFinDigitBits;
+
+struct FinChunk {
+  int begin, end;
+};
+__device__ __forceinline__ FinChunk fin_chunk(int nRW, int totalWaves, int gw) {
+  const int chunk = (((nRW + totalWaves - 1) / totalWaves) + 63) & ~63;
+  FinChunk c;
+  c.begin = min(gw * chunk, nRW);
+  c.end = min(c.begin + chunk, nRW);
+  return c;
+}
+__device__ __forceinline__ unsigned long long fin_digit_peers(bool valid, int dgt) {
+  unsigned long long peers = __ballot(valid);
+#pragma unroll
+  for (int b = 0; b < kFinDigitBits; b++) {
+    const unsigned long long bal = __ballot((dgt >> b) & 1);
+    peers &= ((dgt >> b) & 1) ? bal : ~bal;
+  }
+  return peers;
+}
+__device__ __forceinline__ int fin_passes(int maxC) {
+  int nBits = 0;
+  while ((maxC >> nBits) != 0) nBits++;
+  return (nBits + kFinDigitBits - 1) / kFinDigitBits;
+}
+
+__global__ __launch_bounds__(256) void finalize_partials_kernel(
+    const int32_t* __restrict__ blockPartition, int nRW, int totalWaves,
+    unsigned* __restrict__ waveSum, int* __restrict__ waveMax) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gw >= totalWaves) return;
+  const FinChunk c = fin_chunk(nRW, totalWaves, gw);
+  unsigned sum = 0;
+  int mx = 0;
+  for (int i = c.begin + lane; i < c.end; i += 64) {
+    const int v = blockPartition[i];
+    sum += (unsigned)v;
+    mx = max(mx, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    sum += __shfl_xor(sum, off);
+    mx = max(mx, __shfl_xor(mx, off));
+  }
+  if (lane == 0) {
+    waveSum[gw] = sum;
+    waveMax[gw] = mx;
+  }
+}
+
+// digit histogram of a wave's chunk into hist[gw * 64 + digit]; sBins: 64 LDS counters of the wave
+__device__ __forceinline__ void fin_histogram(const int32_t* __restrict__ keys, bool fromCounts,
+                                              int maxC, FinChunk c, int shift, int lane,
+                                              unsigned* sBins, unsigned* __restrict__ histRow) {
+  sBins[lane] = 0;
+  wave_lds_sync();
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  int keyNext = (c.begin + lane < c.end) ? keys[c.begin + lane] : 0;
+  for (int base = c.begin; base < c.end; base += 64) {
+    const int i = base + lane;
+    const bool valid = i < c.end;
+    const int raw = keyNext;
+    keyNext = (i + 64 < c.end) ? keys[i + 64] : 0;
+    const int key = fromCounts ? maxC - raw : raw;
+    const int dgt = (key >> shift) & (kFinBins - 1);
+    const unsigned long long peers = fin_digit_peers(valid, dgt);
+    // the first lane of every group of equal digits adds the group to its bin
+    if (valid && (peers & ltMask) == 0ull) sBins[dgt] += __popcll(peers);
+  }
+  wave_lds_sync();
+  histRow[lane] = sBins[lane];
+}
+
+__global__ __launch_bounds__(256) void finalize_scan_kernel(
+    const int32_t* __restrict__ blockPartition, int nRW, int totalWaves,
+    const unsigned* __restrict__ waveSum, const int* __restrict__ waveMax,
+    int32_t* __restrict__ rowWindowOffset, unsigned* __restrict__ hist,
+    WsHeader* __restrict__ hdr) {
+  __shared__ unsigned sBins[4][kFinBins];
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gw >= totalWaves) return;
+  const FinChunk c = fin_chunk(nRW, totalWaves, gw);
+  unsigned carry = 0, total = 0;
+  int maxC = 0;
+#pragma unroll 4
+  for (int k = lane; k < totalWaves; k += 64) {
+    const unsigned t = waveSum[k];
+    if (k < gw) carry += t;
+    total += t;
+    maxC = max(maxC, waveMax[k]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    carry += __shfl_xor(carry, off);
+    total += __shfl_xor(total, off);
+    maxC = max(maxC, __shfl_xor(maxC, off));
+  }
+  for (int base = c.begin; base < c.end; base += 64) {
+    const int i = base + lane;
+    const unsigned v = (i < c.end) ? (unsigned)blockPartition[i] : 0u;
+    const unsigned incl = wave_inclusive_scan(v, lane);
+    if (i < c.end) rowWindowOffset[i + 1] = (int)(carry + incl);
+    carry += __shfl(incl, 63);
+  }
+  if (gw == 0 && lane == 0) {
+    rowWindowOffset[0] = 0;
+    hdr->nTcb = (long long)total;
+    hdr->maxCount = maxC;
+  }
+  fin_histogram(blockPartition, true, maxC, c, 0, lane, sBins[threadIdx.x >> 6],
+                hist + (size_t)gw * kFinBins);
+}
+
+__global__ __launch_bounds__(256) void finalize_histogram_kernel(
+    int nRW, int totalWaves, int pass, const int32_t* __restrict__ keysA,
+    const int32_t* __restrict__ keysB, unsigned* __restrict__ hist,
+    const WsHeader* __restrict__ hdr) {
+  __shared__ unsigned sBins[4][kFinBins];
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gw >= totalWaves) return;
+  const int maxC = hdr->maxCount;
+  const int nPass = fin_passes(maxC);
+  if (pass >= nPass) return;
+  // the keys this pass reads are the ones the previous pass wrote
+  const bool prevToOut = ((nPass - pass) & 1) == 0;
+  const int32_t* kSrc = prevToOut ? keysA : keysB;
+  fin_histogram(kSrc, false, maxC, fin_chunk(nRW, totalWaves, gw), pass * kFinDigitBits, lane,
+                sBins[threadIdx.x >> 6], hist + (size_t)gw * kFinBins);
+}
+
+__global__ __launch_bounds__(256) void finalize_scatter_kernel(
+    const int32_t* __restrict__ blockPartition, int nRW, int totalWaves, int pass,
+    int32_t* __restrict__ sortedRowWindows, int32_t* __restrict__ keysA,
+    int32_t* __restrict__ keysB, int32_t* __restrict__ valsTmp, const unsigned* __restrict__ hist,
+    const WsHeader* __restrict__ hdr) {
+  __shared__ unsigned sPos[4][kFinBins];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int gw = blockIdx.x * 4 + wave;
+  if (gw >= totalWaves) return;
+  const FinChunk c = fin_chunk(nRW, totalWaves, gw);
+  const int maxC = hdr->maxCount;
+  const int nPass = fin_passes(maxC);
+  if (nPass == 0) {  // every window is empty: the order is the identity
+    if (pass == 0)
+      for (int i = c.begin + lane; i < c.end; i += 64) sortedRowWindows[i] = i;
+    return;
+  }
+  if (pass >= nPass) return;
+  const int shift = pass * kFinDigitBits;
+  const bool toOut = ((nPass - 1 - pass) & 1) == 0;
+  int32_t* kDst = toOut ? keysA : keysB;
+  int32_t* vDst = toOut ? sortedRowWindows : valsTmp;
+  const int32_t* kSrc = toOut ? keysB : keysA;
+  const int32_t* vSrc = toOut ? valsTmp : sortedRowWindows;
+  // start of (digit = lane, this wave): all smaller digits, then the same digit in earlier waves
+  unsigned digitTotal = 0, before = 0;
+#pragma unroll 8
+  for (int k = 0; k < totalWaves; k++) {
+    const unsigned cnt = hist[(size_t)k * kFinBins + lane];
+    digitTotal += cnt;
+    before += (k < gw) ? cnt : 0u;
+  }
+  const unsigned start = wave_inclusive_scan(digitTotal, lane) - digitTotal + before;
+  sPos[wave][lane] = start;
+  wave_lds_sync();
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
+  auto load_key = [&](int i) {
+    return (i < c.end) ? ((pass == 0) ? (maxC - blockPartition[i]) : kSrc[i]) : 0;
+  };
+  auto load_val = [&](int i) { return (i < c.end) ? ((pass == 0) ? i : vSrc[i]) : 0; };
+  int keyNext = load_key(c.begin + lane);
+  int valNext = load_val(c.begin + lane);
+  for (int base = c.begin; base < c.end; base += 64) {
+    const int i = base + lane;
+    const bool valid = i < c.end;
+    const int key = keyNext, val = valNext;
+    keyNext = load_key(i + 64);
+    valNext = load_val(i + 64);
+    const int dgt = (key >> shift) & (kFinBins - 1);
+    const unsigned long long peers = fin_digit_peers(valid, dgt);
+    if (valid) {
+      const unsigned pos = sPos[wave][dgt] + __popcll(peers & ltMask);
+      kDst[pos] = key;
+      vDst[pos] = val;
+    }
+    // the last peer moves the digit's running position (the wave's LDS accesses stay in order)
+    if (valid && (peers >> lane) == 1ull) sPos[wave][dgt] += __popcll(peers);
+  }
+}
+
 // ------------------------------------------------------------------ phase 2
+// Any window, TC blocks at a time: rows may hold repeated or descending columns. sCnt
+// ([TC * 16]) and sBm ([TC * WPT]) are the caller's LDS; sRow holds the window's 17 row pointers;
+// *sUnsorted must be 0 on entry. Every thread of the workgroup calls this.
 template <int W, int TB, int TC>
-__global__ __launch_bounds__(TB) void window_fill_kernel(
-    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
-    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
-    long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
+__device__ __forceinline__ void fill_window_generic(
+    const int32_t* __restrict__ colIdx, const int32_t* __restrict__ edgeToColumn, int w, int base,
+    int nb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
     int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
-    unsigned long long* __restrict__ bitmap, int minBlocks, int maxBlocks) {
+    unsigned long long* __restrict__ bitmap, unsigned* sCnt, unsigned long long* sBm,
+    const int* sRow, unsigned* sWaveTot, unsigned* sUnsortedPtr) {
   constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
   constexpr int LOGW = (W == 16) ? 4 : 3;
-  __shared__ unsigned sCnt[TC * 16];            // [block][row] counts, then running positions
-  __shared__ unsigned long long sBm[TC * WPT];  // bitmaps of the chunk
-  __shared__ int sRow[17];
-  __shared__ unsigned sWaveTot[TB / 64];
-  __shared__ unsigned sUnsorted;  // bit r: row r's columns are not strictly ascending
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int w = blockIdx.x;
-  if (tid == 0) sUnsorted = 0u;
-  if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
-  const int base = rowWindowOffset[w];
-  const int nb = rowWindowOffset[w + 1] - base;
-  // a launch may be one of two that share the windows by length: [minBlocks, maxBlocks]
-  if (nb == 0 || nb < minBlocks || nb > maxBlocks) return;
-  const int r0 = w * 16;
-  if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
-  __syncthreads();
   const int eS = sRow[0], eE = sRow[16];
   const unsigned long long ltMask = (1ull << lane) - 1ull;
   unsigned carry = (unsigned)eS;  // absolute edge position where the next TC block starts
@@ -624,7 +938,7 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
           const int e = e0 + u * TB;
           if (e < eE && e > eS) {
             const int r = row_of_edge(sRow, e);
-            if (e > sRow[r] && colIdx[e - 1] >= cols[u]) atomicOr(&sUnsorted, 1u << r);
+            if (e > sRow[r] && colIdx[e - 1] >= cols[u]) atomicOr(sUnsortedPtr, 1u << r);
           }
         }
       }
@@ -667,7 +981,7 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
         unsigned run = carry + waveOff + incl - nnz;
         tcblockOffset[gt] = (int)run;
         tcblockRowid[gt] = w;
-        if (sUnsorted == 0u) {
+        if (*sUnsortedPtr == 0u) {
           // Every row of the window is strictly ascending, so the block's tile ids are its set
           // bits read row by row, left to right (src/utils.cu:213-223 walks the edges in that
           // order): this thread writes them all, next to the previous block's.
@@ -723,7 +1037,7 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
     // earlier edges of that row in the block. In a strictly ascending row those are exactly the
     // bits left of the edge's own bit in the block's bitmap row, so every edge of such a row
     // finds its place on its own; the other rows are replayed in order below.
-    const unsigned unsorted = sUnsorted;
+    const unsigned unsorted = *sUnsortedPtr;
     for (int e = eS + tid; unsorted != 0u && e < eE; e += TB) {
       const int ec = edgeToColumn[e];
       const int t = (ec >> LOGW) - tc0;
@@ -770,6 +1084,177 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
   }
 }
 
+
+// One workgroup (or one wave) per window. Windows whose rows are all strictly ascending (every
+// CSR that is sorted and free of repeated entries) take the short way: every edge sets its bit in
+// the LDS bitmaps and drops its column id into the LDS copy of the block's id slots; a block's
+// non-zero count is then the population count of its bitmap, its tile ids are its set bits read
+// row by row (src/utils.cu:213-223 walks the edges in exactly that order), and bitmaps and ids
+// leave LDS as contiguous runs. A window with a repeated or descending column is handed to
+// fill_window_generic. TC blocks of LDS at a time on the short way, TCG on the general one.
+template <int W, int TB, int TC, int TCG>
+__global__ __launch_bounds__(TB) void window_fill_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
+    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
+    long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
+    int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
+    unsigned long long* __restrict__ bitmap, int minBlocks, int maxBlocks) {
+  constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
+  constexpr int LOGW = (W == 16) ? 4 : 3;
+  constexpr int FAST_BYTES = TC * (WPT * 8 + W * 4);
+  constexpr int GEN_BYTES = TCG * (16 * 4 + WPT * 8);
+  constexpr int RAW_BYTES = FAST_BYTES > GEN_BYTES ? FAST_BYTES : GEN_BYTES;
+  __shared__ __align__(16) unsigned char sRaw[RAW_BYTES];
+  __shared__ int sRow[17];
+  __shared__ unsigned sWaveTot[TB / 64];
+  __shared__ unsigned sUnsorted;  // bit r: row r's columns are not strictly ascending
+  unsigned long long* sBm = reinterpret_cast<unsigned long long*>(sRaw);       // [TC * WPT]
+  int32_t* sIds = reinterpret_cast<int32_t*>(sRaw + TC * WPT * 8);             // [TC * W]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int w = blockIdx.x;
+  if (tid == 0) sUnsorted = 0u;
+  if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
+  const int base = rowWindowOffset[w];
+  const int nb = rowWindowOffset[w + 1] - base;
+  // a launch may be one of two that share the windows by length: [minBlocks, maxBlocks]
+  if (nb == 0 || nb < minBlocks || nb > maxBlocks) return;
+  const int r0 = w * 16;
+  if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
+  __syncthreads();
+  const int eS = sRow[0], eE = sRow[16];
+  unsigned carry = (unsigned)eS;  // absolute edge position where the next TC block starts
+
+  for (int tc0 = 0; tc0 < nb; tc0 += TC) {
+    const int nt = min(TC, nb - tc0);
+    for (int i = tid; i < nt * WPT; i += TB) sBm[i] = 0ull;
+    for (int i = tid; i < nt * W; i += TB) sIds[i] = 0;
+    __syncthreads();
+    // Four CONSECUTIVE edges per thread (one 16-byte load of ranks, one of column ids, from a
+    // 16-byte aligned index). Consecutive edges of a row fall into the same bitmap byte (row r
+    // of an 8-column sub-block) up to eight at a time, so a thread first ORs its edges' bits
+    // together per byte and then issues one 32-bit LDS atomic per distinct byte.
+    unsigned* sBmWords = reinterpret_cast<unsigned*>(sBm);
+    for (int e0 = (eS & ~3) + 4 * tid; e0 < eE; e0 += 4 * TB) {
+      int ecs[4], cols[4];
+      if (e0 + 4 <= E) {
+        const int4 a = *reinterpret_cast<const int4*>(edgeToColumn + e0);
+        const int4 b = *reinterpret_cast<const int4*>(colIdx + e0);
+        ecs[0] = a.x; ecs[1] = a.y; ecs[2] = a.z; ecs[3] = a.w;
+        cols[0] = b.x; cols[1] = b.y; cols[2] = b.z; cols[3] = b.w;
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          ecs[u] = (e0 + u < E) ? edgeToColumn[e0 + u] : 0;
+          cols[u] = (e0 + u < E) ? colIdx[e0 + u] : 0;
+        }
+      }
+      int left = (tc0 == 0 && e0 > eS) ? colIdx[e0 - 1] : -1;
+      const int eLo = e0 > eS ? e0 : eS;
+      const int eHi = (e0 + 3 < eE - 1) ? e0 + 3 : eE - 1;
+      const int rLo = row_of_edge(sRow, eLo);
+      const int rHi = row_of_edge(sRow, eHi);
+      int curKey = -1;
+      unsigned curMask = 0;
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int e = e0 + u;
+        const bool valid = e >= eS && e < eE;
+        const int r = (rLo == rHi) ? rLo : (valid ? row_of_edge(sRow, e) : rLo);
+        // once per window: is every edge right of its left neighbour in the same row?
+        if (tc0 == 0 && valid && e > sRow[r] && left >= cols[u]) atomicOr(&sUnsorted, 1u << r);
+        left = cols[u];
+        const int t = (ecs[u] >> LOGW) - tc0;
+        if (valid && (unsigned)t < (unsigned)nt) {
+          const int cl = ecs[u] & (W - 1);
+          sIds[t * W + cl] = cols[u];
+          // 8x8 sub-blocks in column-major order; byte 7 - r%8 of the sub-block's word is row
+          // r%8, MSB first
+          const int sub = (cl >> 3) * (W / 8) + (r >> 3);
+          const int key = (t * WPT + sub) * 8 + 7 - (r & 7);
+          const unsigned m8 = 0x80u >> (cl & 7);
+          if (key == curKey) {
+            curMask |= m8;
+          } else {
+            if (curKey >= 0) atomicOr(&sBmWords[curKey >> 2], curMask << (8 * (curKey & 3)));
+            curKey = key;
+            curMask = m8;
+          }
+        }
+      }
+      if (curKey >= 0) atomicOr(&sBmWords[curKey >> 2], curMask << (8 * (curKey & 3)));
+    }
+    __syncthreads();
+    if (sUnsorted != 0u) break;  // known after the first pass over the window's edges
+    for (int tb = 0; tb < nt; tb += TB) {
+      const int t = tb + tid;
+      unsigned long long words[WPT];
+      unsigned nnz = 0;
+      if (t < nt) {
+#pragma unroll
+        for (int k = 0; k < WPT; k++) {
+          words[k] = sBm[t * WPT + k];
+          nnz += __popcll(words[k]);
+        }
+      }
+      const unsigned incl = wave_inclusive_scan(nnz, lane);
+      if (lane == 63) sWaveTot[wave] = incl;
+      __syncthreads();
+      unsigned waveOff = 0, tileTot = 0;
+#pragma unroll
+      for (int v = 0; v < TB / 64; v++) {
+        const unsigned x = sWaveTot[v];
+        if (v < wave) waveOff += x;
+        tileTot += x;
+      }
+      if (t < nt) {
+        const int64_t gt = (int64_t)base + tc0 + t;
+        unsigned pos = carry + waveOff + incl - nnz;
+        tcblockOffset[gt] = (int)pos;
+        tcblockRowid[gt] = w;
+        // tile ids: the block's set bits read row by row (each lane walks its own block; the
+        // byte stores of neighbouring lanes fall next to each other)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          unsigned rowBits = 0;  // W bits, column 0 in the most significant one
+#pragma unroll
+          for (int h = 0; h < W / 8; h++)
+            rowBits = (rowBits << 8) |
+                      ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
+          while (rowBits) {
+            const int cl = __clz(rowBits) - (32 - W);
+            tcblocktileId[pos++] = (uint8_t)(r * W + cl);
+            rowBits &= ~(1u << (W - 1 - cl));
+          }
+        }
+      }
+      carry += tileTot;
+      __syncthreads();
+    }
+    // bitmaps and column ids of the chunk as contiguous runs (unused id slots stay 0)
+    {
+      unsigned long long* bmDst = bitmap + ((int64_t)base + tc0) * WPT;
+      for (int i = tid; i < nt * WPT; i += TB) bmDst[i] = sBm[i];
+      int32_t* idDst = sparseAToXidx + ((int64_t)base + tc0) * W;
+      for (int i = tid; i < nt * W; i += TB) idDst[i] = sIds[i];
+    }
+    __syncthreads();
+  }
+  if (sUnsorted != 0u) {
+    // repeated or descending columns somewhere in the window: start over on the general way
+    __syncthreads();
+    if (tid == 0) sUnsorted = 0u;
+    __syncthreads();
+    unsigned* gCnt = reinterpret_cast<unsigned*>(sRaw);                                  // [TCG*16]
+    unsigned long long* gBm = reinterpret_cast<unsigned long long*>(sRaw + TCG * 64);    // [TCG*WPT]
+    fill_window_generic<W, TB, TCG>(colIdx, edgeToColumn, w, base, nb, tcblockRowid,
+                                    tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, gCnt, gBm,
+                                    sRow, sWaveTot, &sUnsorted);
+  }
+}
+
 __global__ void set_tail_kernel(int32_t* tcblockOffset, long long nTcb, int E) {
   tcblockOffset[nTcb] = E;
 }
@@ -779,15 +1264,25 @@ __global__ void clear_header_kernel(WsHeader* hdr) {
   hdr->error = 0;
   hdr->nBig = 0;
   hdr->nextBig = 0;
+  hdr->maxCount = 0;
+  hdr->nextMed = 0;
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 }  // namespace
 
+// waves of the multi-workgroup finalize (0: the single-workgroup kernel is used)
+int finalize_waves(int nRW) {
+  if (nRW <= 16384) return 0;
+  const int w = (nRW + 511) / 512;
+  return w < 4096 ? w : 4096;
+}
+
 size_t preprocess_workspace_bytes(int N, int /*E*/) {
   const size_t nRW = (size_t)(N + kWinRows - 1) / kWinRows;
-  return kWsHeaderBytes + 3 * align256(nRW * sizeof(int32_t));
+  const size_t fin = (size_t)finalize_waves((int)nRW) * (2 + kFinBins) * sizeof(int32_t);
+  return kWsHeaderBytes + 3 * align256(nRW * sizeof(int32_t)) + align256(fin);
 }
 
 namespace {
@@ -839,10 +1334,26 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
     }
     F3S_HIP_CHECK(hipGetLastError());
     // eight waves per window when windows are long (more loads and LDS atomics in flight)
+    // queued windows of a few thousand edges on a graph that needs several bitset passes are
+    // sorted instead (window_rank_sort_kernel); the bitset kernel then skips them
+    const bool sortMedium = queue != nullptr && nPasses >= 2;
+    const int skipUpTo = sortMedium ? kMedMax : 0;
+    if (sortMedium) {
+      const int medGrid = nRW < 1024 ? nRW : 1024;
+      if (W == 16)
+        hipLaunchKernelGGL(window_rank_sort_kernel<16>, dim3(medGrid), dim3(kMedThreads), 0,
+                           stream, rowPtr, colIdx, N, colBits, blockPartition, edgeToColumn,
+                           edgeToRow, hdr, queue);
+      else
+        hipLaunchKernelGGL(window_rank_sort_kernel<8>, dim3(medGrid), dim3(kMedThreads), 0, stream,
+                           rowPtr, colIdx, N, colBits, blockPartition, edgeToColumn, edgeToRow,
+                           hdr, queue);
+      F3S_HIP_CHECK(hipGetLastError());
+    }
 #define F3S_RANK(WW, TBB)                                                                     \
   hipLaunchKernelGGL((window_rank_kernel<WW, TBB>), dim3(rankGrid), dim3(TBB), lds, stream,   \
                      rowPtr, colIdx, N, range, nPasses, blockPartition,                       \
-                     edgeToColumn, edgeToRow, hdr, queue)
+                     edgeToColumn, edgeToRow, hdr, queue, skipUpTo)
     // the queue lives in the buffer finalize_count_kernel later uses for its values and is
     // drained by at most 8 workgroups per CU
     const int rankGrid = big ? nRW : (nRW < 2048 ? nRW : 2048);
@@ -854,8 +1365,32 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
 #undef F3S_RANK
     F3S_HIP_CHECK(hipGetLastError());
   }
-  hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
-                     nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
+  const int finWaves = finalize_waves(nRW);
+  if (finWaves == 0) {
+    hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
+                       nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
+    F3S_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
+  unsigned* waveSum = reinterpret_cast<unsigned*>(ws + kWsHeaderBytes + 3 * seg);
+  int* waveMax = reinterpret_cast<int*>(waveSum + finWaves);
+  unsigned* hist = waveSum + 2 * (size_t)finWaves;
+  const dim3 grid((unsigned)((finWaves + 3) / 4)), block(256);
+  hipLaunchKernelGGL(finalize_partials_kernel, grid, block, 0, stream, blockPartition, nRW,
+                     finWaves, waveSum, waveMax);
+  hipLaunchKernelGGL(finalize_scan_kernel, grid, block, 0, stream, blockPartition, nRW, finWaves,
+                     waveSum, waveMax, rowWindowOffset, hist, hdr);
+  // a window holds at most ceil(N / W) blocks: that bounds the passes that can be needed
+  int maxBits = 0;
+  while ((((int64_t)N + W - 1) / W >> maxBits) != 0) maxBits++;
+  const int maxPass = (maxBits + kFinDigitBits - 1) / kFinDigitBits;
+  for (int pass = 0; pass < (maxPass > 0 ? maxPass : 1); pass++) {
+    if (pass > 0)
+      hipLaunchKernelGGL(finalize_histogram_kernel, grid, block, 0, stream, nRW, finWaves, pass,
+                         keysA, keysB, hist, hdr);
+    hipLaunchKernelGGL(finalize_scatter_kernel, grid, block, 0, stream, blockPartition, nRW,
+                       finWaves, pass, sortedRowWindows, keysA, keysB, valsTmp, hist, hdr);
+  }
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -969,27 +1504,27 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
   // of short windows get one wave per window and 128 blocks of LDS, so that a CU works on a
   // dozen windows at once instead of three with most of their waves idle; their few windows of
   // more than 128 blocks are left to a second launch with four waves per window.
-#define F3S_FILL(WW, TBB, TCC, LO, HI)                                                         \
-  hipLaunchKernelGGL((window_fill_kernel<WW, TBB, TCC>), dim3(nRW), dim3(TBB), 0, stream,      \
+#define F3S_FILL(WW, TBB, TCC, TCG, LO, HI)                                                    \
+  hipLaunchKernelGGL((window_fill_kernel<WW, TBB, TCC, TCG>), dim3(nRW), dim3(TBB), 0, stream, \
                      rowPtr, colIdx, N, E, edgeToColumn, rowWindowOffset, (long long)nTcb,     \
                      tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx, bm, LO, HI)
   const bool big = (int64_t)E >= (int64_t)nRW * 2048;
   constexpr int kAll = 0x7FFFFFFF;
   if (W == 16) {
     if (big) {
-      F3S_FILL(16, 512, kFillChunk, 0, kAll);
+      F3S_FILL(16, 512, kFillChunk, kFillChunkGeneric, 0, kAll);
     } else {
-      F3S_FILL(16, 64, kFillChunkSmall, 0, kFillChunkSmall);
+      F3S_FILL(16, 64, kFillChunkSmall, kFillChunkSmall, 0, kFillChunkSmall);
       F3S_HIP_CHECK(hipGetLastError());
-      F3S_FILL(16, 256, kFillChunk, kFillChunkSmall + 1, kAll);
+      F3S_FILL(16, 256, kFillChunk, kFillChunkGeneric, kFillChunkSmall + 1, kAll);
     }
   } else {
     if (big) {
-      F3S_FILL(8, 512, kFillChunk, 0, kAll);
+      F3S_FILL(8, 512, kFillChunk, kFillChunkGeneric, 0, kAll);
     } else {
-      F3S_FILL(8, 64, kFillChunkSmall, 0, kFillChunkSmall);
+      F3S_FILL(8, 64, kFillChunkSmall, kFillChunkSmall, 0, kFillChunkSmall);
       F3S_HIP_CHECK(hipGetLastError());
-      F3S_FILL(8, 256, kFillChunk, kFillChunkSmall + 1, kAll);
+      F3S_FILL(8, 256, kFillChunk, kFillChunkGeneric, kFillChunkSmall + 1, kAll);
     }
   }
 #undef F3S_FILL

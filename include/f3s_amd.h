@@ -70,7 +70,7 @@ int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, in
  *   - the scratch is a buffer the library owns, a static device array of
  *     f3s_preprocess_static_scratch_bytes() = 8 MiB per GPU that lives until the process ends;
  *     graphs needing more (f3s_preprocess_workspace_bytes(N, E) > 8 MiB, i.e. above about
- *     11.1 million nodes) are rejected with status -5 and a message;
+ *     10.7 million nodes) are rejected with status -5 and a message;
  *   - nothing is copied to the host and the stream is not synchronised: result_dev is a DEVICE
  *     pointer to two int64, out: {total TC blocks, 1 if a column index lay outside [0, N) else 0}.
  * The call makes no hipMalloc / hipFree and uses no allocating library routine; everything is

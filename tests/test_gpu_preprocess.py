@@ -115,6 +115,29 @@ def test_more_than_4m_nodes_takes_the_bitonic_short_window_kernel(oracle_mod):
     compare_preprocess(got, want)
 
 
+def test_many_windows_three_sorting_passes_and_all_empty(oracle_mod):
+    """More than 16384 windows: the scan and the window order run over many workgroups. One hub
+    window of more than 4095 TC blocks makes the order take three 6-bit passes; most windows tie
+    at 0 or 1 blocks (ties keep ascending window id). Then the same size with no edge at all."""
+    print("case many_windows", flush=True)
+    N = 400_000
+    rng = np.random.default_rng(5)
+    deg = np.zeros(N, np.int64)
+    some = rng.choice(N, size=60_000, replace=False)
+    deg[some] = rng.integers(1, 30, size=len(some))
+    deg[200_000:200_016] = 6_000  # 16 hub rows in one window: ~90k distinct columns
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(deg)
+    colIdx = rng.integers(0, N, size=int(rowPtr[-1])).astype(np.int32)
+    got = run_gpu(rowPtr, colIdx, N)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
+    assert want["blockPartition"].max() > 4095
+    compare_preprocess(got, want)
+    got = run_gpu(np.zeros(N + 1, np.int32), np.zeros(0, np.int32), N)
+    assert got["blockCount"] == 0 and not got["rowWindowOffset"].any()
+    assert np.array_equal(got["sortedRowWindows"], np.arange((N + 15) // 16))
+
+
 def test_empty_graph_and_tiny():
     print("case empty", flush=True)
     got = run_gpu(np.zeros(41, np.int32), np.zeros(0, np.int32), 40)
