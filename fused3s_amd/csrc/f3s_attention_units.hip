@@ -20,6 +20,8 @@
 // is kept: units are issued heavy windows first.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "f3s_common.h"
 #include "f3s_pair_pipeline.h"
 
@@ -32,14 +34,17 @@ using pipe::uniform;
 constexpr int kXcds = 8;
 constexpr int kMaxPhases = 16;
 constexpr int kUnitWaves = 4;  // waves (= units) per workgroup; they do not cooperate
+constexpr int kQueueBatch = 8;  // units a persistent wave takes per visit to a queue
 
 // sliceStart[w * (S + 1) + s] = first TC block of window w whose first (smallest) column id is
 // >= s * sliceWidth; entry S is the window's end. One thread per entry, binary search over the
 // window's blocks (their first columns ascend).
 __global__ void slice_index_kernel(const int32_t* __restrict__ rowWindowOffset,
                                    const int32_t* __restrict__ sparseAToXidx, int nRW, int S,
-                                   int sliceWidth, int32_t* __restrict__ sliceStart) {
+                                   int sliceWidth, int32_t* __restrict__ sliceStart,
+                                   int32_t* __restrict__ cursors) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < kXcds) cursors[idx] = 0;  // work queues of f3s_fwd_sliced_kernel
   const int per = S + 1;
   if (idx >= (int64_t)nRW * per) return;
   const int w = (int)(idx / per), b = (int)(idx % per);
@@ -173,6 +178,93 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
   }
 }
 
+// The column-sliced schedule with persistent waves and work queues, the form that does not lean
+// on how the hardware deals workgroups to XCDs or on the order in which it starts them. The grid
+// is a fixed number of workgroups (as many as fit the CUs); every wave pulls (window, slice) units
+// from a queue per XCD until all are done: queue x holds the units of slices x, x + 8, ... in
+// heavy-first window order, phase by phase, and a wave serves the queue of the XCD it runs on
+// (read from the hardware, XCC_ID) before it helps out on the others.
+// Measured on the 233k-node benchmark graph (d = 64): 1.72 ms with eight units per queue visit,
+// 2.0 ms with one (a device-wide atomic is served on the memory side and one address takes about
+// ten million of them per second), against 1.54 ms for f3s_fwd_unit_kernel, where the launch order
+// is the schedule. It is therefore the fallback, used when workgroups turn out not to be dealt
+// round-robin to the XCDs (xcd_round_robin, below), or on request (F3S_SLICED_PERSISTENT=1).
+template <typename ET, int D, bool SOFTMAX>
+__global__ __launch_bounds__(kUnitWaves * 64)
+__attribute__((amdgpu_waves_per_eu(unit_waves_per_simd(D), unit_waves_per_simd(D)))) void
+f3s_fwd_sliced_kernel(const int32_t* __restrict__ windowOrder,
+                      const int32_t* __restrict__ sparseAToXidx,
+                      const uint8_t* __restrict__ bitmapBytes,
+                      const int32_t* __restrict__ sliceStart, int32_t* __restrict__ cursors, int S,
+                      int P, int N, int nRW, int64_t nTcb, const ET* __restrict__ Q,
+                      const ET* __restrict__ K, const ET* __restrict__ V, float scaleLog2,
+                      float* __restrict__ partial) {
+  typedef pipe::PairPipeline<ET, D, SOFTMAX, false, false> Pipe;
+  constexpr int T = D / 16;
+  extern __shared__ __align__(1024) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  unsigned xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  const int home = (int)(xcc & (kXcds - 1));
+
+  pipe::Problem<ET> pb;
+  pb.sparseAToXidx = sparseAToXidx;
+  pb.bitmapBytes = bitmapBytes;
+  pb.Q = Q;
+  pb.K = K;
+  pb.V = V;
+  pb.N = N;
+  pb.scaleLog2 = scaleLog2;
+  pb.pitchIn = D;
+  pb.nTcb = nTcb;
+  pb.sddmm = nullptr;
+  const unsigned ringAddr =
+      (unsigned)(uintptr_t)(F3S_LDS unsigned char*)smem + (unsigned)wave * pipe::Geo<D>::WAVE_BYTES;
+  const int total = P * nRW;  // units per queue (empty ones included)
+  int batchNext = 0, batchLeft = 0;
+  for (int k = 0; k < kXcds; k++) {
+    const int x = (home + k) & (kXcds - 1);
+    while (true) {
+      int u = 0;
+      // a device-wide atomic is served on the memory side (the XCDs' L2s are not coherent
+      // with each other): a wave takes kQueueBatch units per visit to keep the queue's address
+      // from becoming the bottleneck
+      if (batchLeft == 0) {
+        if (lane == 0) batchNext = atomicAdd(&cursors[x], kQueueBatch);
+        batchNext = uniform(batchNext);
+        batchLeft = kQueueBatch;
+      }
+      u = batchNext++;
+      batchLeft--;
+      if (u >= total) {
+        batchLeft = 0;
+        break;
+      }
+      const int phase = u / nRW;
+      const int pos = u - phase * nRW;
+      const int slice = phase * kXcds + x;
+      const int w = uniform(windowOrder ? windowOrder[pos] : pos);
+      if ((unsigned)w >= (unsigned)nRW) continue;  // a corrupt order entry is not followed
+      const int t0 = uniform(sliceStart[(int64_t)w * (S + 1) + slice]);
+      const int t1 = uniform(sliceStart[(int64_t)w * (S + 1) + slice + 1]);
+      if (t1 <= t0) continue;  // empty unit: nothing is written, the merge skips it
+      if (t0 < 0 || (int64_t)t1 > nTcb) continue;
+      Pipe pp;
+      pp.init(pb, w, ringAddr, 0);
+      pp.run(pb, t0, t1);
+      float* dst = partial + ((int64_t)w * S + slice) * partial_dwords<D>() + lane;
+#pragma unroll
+      for (int jj = 0; jj < T; jj++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          __builtin_nontemporal_store(pp.o[jj][i], dst + (jj * 4 + i) * 64);
+      __builtin_nontemporal_store(pp.m, dst + (D / 4) * 64);
+      __builtin_nontemporal_store(pp.l, dst + (D / 4 + 1) * 64);
+    }
+  }
+}
+
 // One wave per window: log-sum-exp merge of the window's unit partials, then the window's rows.
 // Lane (g, c) holds O[q = c][16j + 4g + i] in O[j * 4 + i], as in the unit kernel.
 template <int D, bool SOFTMAX>
@@ -246,10 +338,8 @@ int allow_lds(KernelT kernel, size_t bytes) {
 // shorter units cost more than their higher hit rate returns (measured 1.99 / 2.23 / 2.48 ms at
 // P = 1 / 2 / 3). F3S_SLICE_PHASES in the environment overrides the choice.
 int choose_phases(int N, int d) {
-  static const int forced = [] {
-    const char* e = getenv("F3S_SLICE_PHASES");
-    return e ? atoi(e) : 0;
-  }();
+  const char* e = getenv("F3S_SLICE_PHASES");  // read per call: tests walk through the phases
+  const int forced = e ? atoi(e) : 0;
   if (forced > 0) return forced > kMaxPhases ? kMaxPhases : forced;
   const int64_t bytes = (int64_t)N * d * 4;  // K + V
   const int64_t perPhase = (int64_t)kXcds * 8 * 1024 * 1024;
@@ -259,18 +349,80 @@ int choose_phases(int N, int d) {
   return P;
 }
 
+// f3s_fwd_unit_kernel's slice-to-XCD mapping assumes that workgroup b of a launch runs on XCD
+// b % 8. That is how the hardware deals workgroups in the partition mode with all eight XCDs
+// behind one device; it is checked once per process and device with a 64-workgroup launch that
+// records XCC_ID (into `scratch64`, 64 ints of the caller's workspace). Returns 0 in *ok when the
+// assumption does not hold; the queue-based kernel is then used.
+__global__ void xcd_probe_kernel(int32_t* __restrict__ out) {
+  unsigned xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(xcc & 0xFu);
+}
+
+int xcd_round_robin(int32_t* scratch64, hipStream_t stream, int* ok) {
+  constexpr int kMaxDev = 64;
+  static std::mutex mu;
+  static int known[kMaxDev] = {};  // 0 unknown, 1 round-robin, 2 not
+  int dev = 0;
+  F3S_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDev) {
+    *ok = 0;
+    return 0;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (known[dev] == 0) {
+    int32_t host[64];
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(64), dim3(64), 0, stream, scratch64);
+    F3S_HIP_CHECK(hipGetLastError());
+    F3S_HIP_CHECK(hipMemcpyAsync(host, scratch64, sizeof(host), hipMemcpyDeviceToHost, stream));
+    F3S_HIP_CHECK(hipStreamSynchronize(stream));
+    bool rr = true;
+    for (int b = 0; b < 64; b++) rr = rr && host[b] == b % kXcds;
+    known[dev] = rr ? 1 : 2;
+  }
+  *ok = known[dev] == 1;
+  return 0;
+}
+
 template <typename ET, int D, bool SOFTMAX>
 int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* atox,
                     const uint64_t* bitmap, int N, const void* Q, const void* K, const void* V,
-                    float scaleLog2, float* out, int32_t* sliceStart, float* partial, int P,
-                    int64_t nTcb, hipStream_t stream) {
+                    float scaleLog2, float* out, int32_t* sliceStart, int32_t* cursors,
+                    float* partial, int P, int64_t nTcb, hipStream_t stream) {
   const int nRW = (N + kWinRows - 1) / kWinRows;
   const int S = P * kXcds;
   const int sliceWidth = (N + S - 1) / S;
   const int64_t entries = (int64_t)nRW * (S + 1);
+  const char* env = getenv("F3S_SLICED_PERSISTENT");
+  const int forced = env ? (env[0] == '0' ? -1 : 1) : 0;
+  bool persistent = forced > 0;
+  if (forced == 0) {  // before the index kernel: the check borrows the cursors' memory
+    int rr = 0;
+    if (int rc = xcd_round_robin(cursors, stream, &rr)) return rc;
+    persistent = rr == 0;
+  }
   hipLaunchKernelGGL(slice_index_kernel, dim3((unsigned)((entries + 255) / 256)), dim3(256), 0,
-                     stream, rwo, atox, nRW, S, sliceWidth, sliceStart);
+                     stream, rwo, atox, nRW, S, sliceWidth, sliceStart, cursors);
   F3S_HIP_CHECK(hipGetLastError());
+  if (persistent) {
+    constexpr size_t ldsP = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES;
+    auto kernel = f3s_fwd_sliced_kernel<ET, D, SOFTMAX>;
+    if (int rc = allow_lds(kernel, ldsP)) return rc;
+    int dev = 0, cus = 0;
+    F3S_HIP_CHECK(hipGetDevice(&dev));
+    F3S_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int perCu = (int)((160 * 1024) / ldsP) > 0 ? (int)((160 * 1024) / ldsP) : 1;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(cus * perCu)), dim3(kUnitWaves * 64), ldsP, stream,
+                       order, atox, reinterpret_cast<const uint8_t*>(bitmap), sliceStart, cursors,
+                       S, P, N, nRW, nTcb, static_cast<const ET*>(Q), static_cast<const ET*>(K),
+                       static_cast<const ET*>(V), scaleLog2, partial);
+    F3S_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL((f3s_merge_slices_kernel<D, SOFTMAX>), dim3((unsigned)((nRW + 3) / 4)),
+                       dim3(256), 0, stream, sliceStart, S, N, nRW, partial, out);
+    F3S_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
   const int nGroups = (nRW + kUnitWaves - 1) / kUnitWaves;
 #ifdef F3S_PROBE_LDS_PAD
   constexpr size_t lds = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES + F3S_PROBE_LDS_PAD;
@@ -298,7 +450,7 @@ size_t attention_sliced_workspace_bytes(int N, int d) {
   const int P = choose_phases(N, d);
   const size_t nRW = (size_t)(N + kWinRows - 1) / kWinRows;
   const size_t S = (size_t)P * kXcds;
-  return align256(nRW * (S + 1) * sizeof(int32_t)) + nRW * S * (size_t)(d / 4 + 2) * 64 * 4;
+  return align256(nRW * (S + 1) * sizeof(int32_t)) + 256 + nRW * S * (size_t)(d / 4 + 2) * 64 * 4;
 }
 
 int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windowOrder,
@@ -311,19 +463,21 @@ int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windo
                 attention_sliced_workspace_bytes(N, d));
   const int P = choose_phases(N, d);
   const size_t nRW = (size_t)(N + kWinRows - 1) / kWinRows;
+  // layout: slice boundaries | the eight queue cursors (256 bytes) | partial results
   int32_t* sliceStart = static_cast<int32_t*>(workspace);
-  float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) +
-                                            align256(nRW * ((size_t)P * kXcds + 1) * 4));
+  const size_t indexBytes = align256(nRW * ((size_t)P * kXcds + 1) * 4);
+  int32_t* cursors = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + indexBytes);
+  float* partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + indexBytes + 256);
 #define F3S_SLICED(ET, DD)                                                                     \
   case DD:                                                                                     \
     return applySoftmax ? launch_sliced_d<ET, DD, true>(rowWindowOffset, windowOrder,          \
                                                         sparseAToXidx, bitmap, N, Q, K, V,     \
-                                                        scaleLog2, out, sliceStart, partial,   \
-                                                        P, nTcb, stream)                       \
+                                                        scaleLog2, out, sliceStart, cursors,   \
+                                                        partial, P, nTcb, stream)              \
                         : launch_sliced_d<ET, DD, false>(rowWindowOffset, windowOrder,         \
                                                          sparseAToXidx, bitmap, N, Q, K, V,    \
-                                                         scaleLog2, out, sliceStart, partial,  \
-                                                         P, nTcb, stream);
+                                                         scaleLog2, out, sliceStart, cursors,  \
+                                                         partial, P, nTcb, stream);
   if (dtype == 0) {
     switch (d) {
       F3S_SLICED(_Float16, 32)

@@ -136,6 +136,30 @@ def test_end_to_end_hip_preprocess_then_attention(oracle_mod):
     assert np.abs(got - txt).max() < MAX_ABS and mean_rel(got, txt) < MEAN_REL
 
 
+@pytest.mark.parametrize("persistent", ["0", "1"])
+@pytest.mark.parametrize("phases", [2, 3])
+def test_column_sliced_schedule_with_several_phases(oracle_mod, monkeypatch, phases, persistent):
+    """16 and 24 column slices (two and three per XCD, which the library only picks by itself above
+    64 MiB of K + V) through the launch-ordered kernel and through the queue-based one."""
+    print("case sliced phases=%d persistent=%s" % (phases, persistent), flush=True)
+    from fused3s_amd import synth
+    monkeypatch.setenv("F3S_SLICE_PHASES", str(phases))
+    monkeypatch.setenv("F3S_SLICED_PERSISTENT", persistent)
+    rp, ci = synth.make_graph("cfg3_chunglu_233k", scale=0.145)
+    N = rp.numel() - 1
+    rng = np.random.default_rng(phases)
+    d = 64
+    Q, K, V = feats(rng, N, d)
+    pre = oracle_mod.preprocess(rp.numpy(), ci.numpy(), N)
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, Q, K, V, 8.0)
+    for order in (pre["sortedRowWindows"], None):
+        got = gpu_attention(pre, N, Q, K, V, 8.0, order, sliced=True)
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() < MAX_ABS
+        assert mean_rel(got, want) < MEAN_REL
+
+
 @pytest.mark.parametrize("d", [32, 64])
 def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
     """The column-sliced schedule on a dense power-law graph (>= 2048 windows, >= 64 TC blocks per
