@@ -2,6 +2,7 @@
 
     python -m fused3s_amd.build            # build both
     python -m fused3s_amd.build --lib      # only libf3s_amd.so
+    python -m fused3s_amd.build --probe gather_only    # a probe library, see PROBES
 
 hipcc cross-compiles for gfx950 without a GPU; the built files stay next to the package so
 that they travel with the source tree.
@@ -22,6 +23,36 @@ HIP_FLAGS = [
     # packed-fp32 code generation is switched off for every device translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+
+# Probe builds: the same sources with one part of the attention step compiled out, to time what
+# is left (their results are wrong on purpose). A probe library goes to
+# fused3s_amd/probes/libf3s_amd_<name>.so and is used by pointing F3S_AMD_LIB at it, e.g.
+#     F3S_AMD_LIB=fused3s_amd/probes/libf3s_amd_gather_only.so python bench.py --no-cpu-baseline
+PROBES = {
+    # K/V rows and metadata are gathered into LDS, nothing reads them back, no arithmetic
+    "gather_only": ["-DF3S_PROBE_NO_COMPUTE", "-DF3S_PROBE_NO_READ"],
+    # the same with every gathered row taken from the first 16384 rows (2 MiB of K, 2 MiB of V:
+    # always an L2 hit) or the first 128 rows (always an L1 hit)
+    "gather_only_l2_rows": ["-DF3S_PROBE_NO_COMPUTE", "-DF3S_PROBE_NO_READ",
+                            "-DF3S_PROBE_ROWMASK=16383"],
+    "gather_only_l1_rows": ["-DF3S_PROBE_NO_COMPUTE", "-DF3S_PROBE_NO_READ",
+                            "-DF3S_PROBE_ROWMASK=127"],
+    # gather and LDS reads, no arithmetic
+    "no_compute": ["-DF3S_PROBE_NO_COMPUTE"],
+    # LDS reads and arithmetic on whatever the first two steps left in the ring, no gather
+    "no_gather": ["-DF3S_PROBE_NO_GATHER"],
+}
+
+
+def build_probe(name):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
+    out_dir = os.path.join(HERE, "probes")
+    os.makedirs(out_dir, exist_ok=True)
+    out = os.path.join(out_dir, "libf3s_amd_%s.so" % name)
+    _run([hipcc] + HIP_FLAGS + PROBES[name] + ["-o", out] + srcs)
+    return out
 
 
 def _run(cmd):
@@ -63,6 +94,11 @@ def build_extension():
 
 
 def main(argv):
+    if "--probe" in argv:
+        names = argv[argv.index("--probe") + 1:] or sorted(PROBES)
+        for name in names:
+            print("built", build_probe(name))
+        return
     build_library()
     print("built", LIB_PATH)
     if "--lib" not in argv and os.path.exists(os.path.join(CSRC, "f3s_torch.cpp")):

@@ -14,6 +14,7 @@
 #include <fstream>
 #include <iomanip>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -209,7 +210,18 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
   const bool sliced = !L.timerFile && f3s_attention_uses_workspace(
                                           nNodes, sparseAToXidx.numel() / 16, (int)d, dtype) != 0;
   const size_t wsBytes = sliced ? f3s_attention_workspace_bytes(nNodes, (int)d) : 0;
-  auto workspace = torch::empty({(int64_t)std::max<size_t>(wsBytes, 4)}, f32.dtype(torch::kUInt8));
+  // one scratch tensor per device, kept between calls and grown when a call needs more; every
+  // entry point blocks until its kernels are done (see timed_launch), so calls cannot overlap
+  static std::mutex wsMutex;
+  static std::map<int, torch::Tensor> wsCache;
+  torch::Tensor workspace;
+  if (sliced) {
+    std::lock_guard<std::mutex> lock(wsMutex);
+    torch::Tensor& cached = wsCache[(int)Q.device().index()];
+    if (!cached.defined() || (size_t)cached.numel() < wsBytes)
+      cached = torch::empty({(int64_t)wsBytes}, f32.dtype(torch::kUInt8));
+    workspace = cached;
+  }
   const float ms = timed_launch("f3s_attention_fwd", [&](void* stream) {
     return f3s_attention_fwd(
         rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,

@@ -2,7 +2,7 @@
  * f3s_amd.h -- C ABI of the MI355X (gfx950) Fused3S library, libf3s_amd.so.
  *
  * Plain pointers and sizes only. Unless stated otherwise every pointer is DEVICE memory on the
- * current HIP device, int32 arrays are 4-byte aligned, sparseAToXidx / Q / K / V / out are
+ * current HIP device, int32 arrays are 4-byte aligned, sparseAToXidx / tcbBitMap / Q / K / V / out are
  * 16-byte aligned, and `stream` is a hipStream_t passed as void* (NULL = default stream).
  * Every entry point returns 0 on success and a negative code on failure; the message is then
  * available from f3s_last_error() (per thread). Nothing here calls exit(): the reference's
@@ -118,7 +118,9 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  *   N, nTCB, d                     nodes; TC blocks (rowWindowOffset[nRW]); head dimension
  *                                  (32, 64 or 128)
  *   dtype                          F3S_DTYPE_F16 (the reference's only type) or F3S_DTYPE_BF16
- *                                  (bf16 MFMA; the probabilities are then rounded to bf16)
+ *                                  (bf16 MFMA; the probabilities then enter the second product as
+ *                                  the sum of two bf16 terms, 16 bits of mantissa instead of the
+ *                                  11 of the reference's fp16 rounding)
  *   Q, K, V [N*d]                  row-major, contiguous
  *   scalingFactor                  unmasked scores are DIVIDED by it (src/F3S_kernel.cu:1666-1667);
  *                                  1.0 = unscaled (:612-613)
@@ -143,8 +145,8 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
 
 /*
  * Bytes of device scratch f3s_attention_fwd can use for a graph of N nodes at head dimension d
- * (slice boundaries per window plus one partial (m, l, O) per window and slice: about
- * 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers
+ * (slice boundaries per window, 256 bytes of queue cursors, plus one partial (m, l, O) per window
+ * and slice: about 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers
  * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);
