@@ -1,6 +1,7 @@
-// Fused 3S attention with one wave per unit of work (gfx950). Same arithmetic per TC-block pair
-// as f3s_fwd_kernel (f3s_attention.hip, which documents the register dataflow and the numerics);
-// what differs is the decomposition. Two uses of the one kernel, f3s_fwd_unit_kernel:
+// Fused 3S attention with one wave per unit of work (gfx950). The step over a TC-block pair is
+// the one every attention kernel here runs (f3s_pair_pipeline.h documents its data flow and its
+// numerics); what differs from the workgroup-per-window kernel of f3s_attention.hip is the
+// decomposition. Two uses of the one kernel, f3s_fwd_unit_kernel:
 //
 // Column-sliced schedule, for graphs with long windows:
 //   * the column range is cut into S = 8 * P slices. Workgroup b runs on XCD b % 8 (the hardware
