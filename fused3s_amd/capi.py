@@ -17,7 +17,8 @@ EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes"
            "f3s_preprocess_count", "f3s_preprocess_fill", "f3s_attention_fwd",
            "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads",
            "f3s_attention_fwd_tcb8", "f3s_attention_uses_workspace",
-           "f3s_preprocess_static_scratch_bytes", "f3s_preprocess_count_static"]
+           "f3s_preprocess_static_scratch_bytes", "f3s_preprocess_count_static",
+           "f3s_preprocess_capacity", "f3s_preprocess"]
 
 
 def lib():
@@ -43,6 +44,12 @@ def lib():
         L.f3s_preprocess_fill.restype = ci
         L.f3s_preprocess_fill.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, ctypes.c_int64, vp, vp,
                                           vp, vp, vp, vp]
+        L.f3s_preprocess_capacity.restype = ctypes.c_int64
+        L.f3s_preprocess_capacity.argtypes = [ci, ctypes.c_int64, ci]
+        L.f3s_preprocess.restype = ci
+        L.f3s_preprocess.argtypes = [vp, vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, ctypes.c_int64,
+                                     vp, vp, vp, vp, vp, vp, cs, ctypes.POINTER(ctypes.c_int64),
+                                     vp]
         L.f3s_attention_fwd.restype = ci
         L.f3s_attention_fwd.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, vp, vp, vp,
                                         ctypes.c_float, ci, vp, vp, vp, cs, vp]
@@ -83,8 +90,13 @@ def _dev(t, dtype, name):
         raise RuntimeError("%s must be contiguous" % name)
 
 
-def preprocess(rowPtr, colIdx, N, H=16, W=16):
-    """Both preprocessing phases through the C ABI. Returns a dict of device tensors."""
+def preprocess(rowPtr, colIdx, N, H=16, W=16, two_phase=False):
+    """Preprocessing through the C ABI. Returns a dict of device tensors.
+
+    Default: f3s_preprocess, one call with the block arrays allocated for
+    f3s_preprocess_capacity(N, E, W) blocks; the returned block tensors are views of their first
+    blockCount entries. two_phase=True: f3s_preprocess_count, exact allocations, then
+    f3s_preprocess_fill (the reference's sequence, src/F3S.cpp:40-87)."""
     L = lib()
     _dev(rowPtr, torch.int32, "rowPtr")
     _dev(colIdx, torch.int32, "colIdx")
@@ -100,20 +112,36 @@ def preprocess(rowPtr, colIdx, N, H=16, W=16):
     wsBytes = L.f3s_preprocess_workspace_bytes(N, E)
     ws = torch.empty(wsBytes, dtype=torch.uint8, device=dev)
     nTcb = ctypes.c_int64(-1)
+    tile = torch.empty(E, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _check(L.f3s_preprocess_count(_ptr(rowPtr), _ptr(colIdx), N, E, H, W,
-                                      _ptr(blockPartition), _ptr(edgeToColumn), _ptr(edgeToRow),
-                                      _ptr(rwo), _ptr(order), _ptr(ws), wsBytes,
-                                      ctypes.byref(nTcb), _stream()))
-        nT = int(nTcb.value)
-        rowid = torch.empty(nT, **i32)
-        tile = torch.empty(E, dtype=torch.uint8, device=dev)
-        toff = torch.empty(nT + 1, **i32)
-        atox = torch.empty(nT * W, **i32)
-        bm = torch.empty(nT * H * W // 64, dtype=torch.uint64, device=dev)
-        _check(L.f3s_preprocess_fill(_ptr(rowPtr), _ptr(colIdx), N, E, H, W, _ptr(edgeToColumn),
-                                     _ptr(rwo), nT, _ptr(rowid), _ptr(tile), _ptr(toff),
-                                     _ptr(atox), _ptr(bm), _stream()))
+        if two_phase:
+            _check(L.f3s_preprocess_count(_ptr(rowPtr), _ptr(colIdx), N, E, H, W,
+                                          _ptr(blockPartition), _ptr(edgeToColumn),
+                                          _ptr(edgeToRow), _ptr(rwo), _ptr(order), _ptr(ws),
+                                          wsBytes, ctypes.byref(nTcb), _stream()))
+            nT = int(nTcb.value)
+            rowid = torch.empty(nT, **i32)
+            toff = torch.empty(nT + 1, **i32)
+            atox = torch.empty(nT * W, **i32)
+            bm = torch.empty(nT * H * W // 64, dtype=torch.uint64, device=dev)
+            _check(L.f3s_preprocess_fill(_ptr(rowPtr), _ptr(colIdx), N, E, H, W,
+                                         _ptr(edgeToColumn), _ptr(rwo), nT, _ptr(rowid),
+                                         _ptr(tile), _ptr(toff), _ptr(atox), _ptr(bm), _stream()))
+        else:
+            cap = int(L.f3s_preprocess_capacity(N, E, W))
+            rowid = torch.empty(cap, **i32)
+            toff = torch.empty(cap + 1, **i32)
+            atox = torch.empty(cap * W, **i32)
+            bm = torch.empty(cap * H * W // 64, dtype=torch.uint64, device=dev)
+            _check(L.f3s_preprocess(_ptr(rowPtr), _ptr(colIdx), N, E, H, W, _ptr(blockPartition),
+                                    _ptr(edgeToColumn), _ptr(edgeToRow), _ptr(rwo), _ptr(order),
+                                    cap, _ptr(rowid), _ptr(tile), _ptr(toff), _ptr(atox),
+                                    _ptr(bm), _ptr(ws), wsBytes, ctypes.byref(nTcb), _stream()))
+            nT = int(nTcb.value)
+            rowid = rowid[:nT]
+            toff = toff[:nT + 1]
+            atox = atox[:nT * W]
+            bm = bm[:nT * H * W // 64]
     return dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
                 tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox, tcbBitMap=bm,
                 blockCount=nT, blockPartition=blockPartition, edgeToColumn=edgeToColumn,

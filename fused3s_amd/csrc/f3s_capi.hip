@@ -89,6 +89,37 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
                                      sparseAToXidx, tcbBitMap, static_cast<hipStream_t>(stream));
 }
 
+int64_t f3s_preprocess_capacity(int N, int64_t E, int W) {
+  if (N < 0) N = 0;
+  if (E < 0) E = 0;
+  if (W != 8) W = 16;
+  return f3s::preprocess_capacity(N, E, W);
+}
+
+int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                   int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                   int32_t* rowWindowOffset, int32_t* sortedRowWindows, int64_t capacity,
+                   int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                   int32_t* sparseAToXidx, uint64_t* tcbBitMap, void* workspace, size_t ws_bytes,
+                   int64_t* nTCB_host, void* stream) {
+  if (!rowPtr || !rowWindowOffset || !workspace || !nTCB_host || !tcblockOffset)
+    return f3s::fail(-1, "f3s_preprocess: null pointer");
+  if (N > 0 && (!blockPartition || !sortedRowWindows))
+    return f3s::fail(-1, "f3s_preprocess: null window output");
+  if (E > 0 && (!colIdx || !edgeToColumn || !edgeToRow || !tcblocktileId || !tcblockRowid ||
+                !sparseAToXidx || !tcbBitMap))
+    return f3s::fail(-1, "f3s_preprocess: null edge or block array");
+  if (f3s::misaligned(workspace, 256))
+    return f3s::fail(-1, "f3s_preprocess: workspace must be 256-byte aligned");
+  if (f3s::misaligned(tcbBitMap, 8))
+    return f3s::fail(-1, "f3s_preprocess: tcbBitMap must be 8-byte aligned");
+  return f3s::launch_preprocess(rowPtr, colIdx, N, E, H, W, blockPartition, edgeToColumn,
+                                edgeToRow, rowWindowOffset, sortedRowWindows, capacity,
+                                tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx,
+                                tcbBitMap, workspace, ws_bytes, nTCB_host,
+                                static_cast<hipStream_t>(stream));
+}
+
 size_t f3s_attention_workspace_bytes(int N, int d) {
   if (N < 0) N = 0;
   if (d < 32) d = 32;

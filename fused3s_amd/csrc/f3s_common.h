@@ -75,4 +75,12 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
                            int32_t* tcblockOffset, int32_t* sparseAToXidx, uint64_t* bitmap,
                            hipStream_t stream);
 
+int64_t preprocess_capacity(int N, int64_t E, int W);
+int launch_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                      int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                      int32_t* rowWindowOffset, int32_t* sortedRowWindows, int64_t capacity,
+                      int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                      int32_t* sparseAToXidx, uint64_t* bitmap, void* workspace, size_t wsBytes,
+                      int64_t* nTcbHost, hipStream_t stream);
+
 }  // namespace f3s

@@ -65,12 +65,16 @@ struct WsHeader {
 };
 constexpr size_t kWsHeaderBytes = 256;
 
-__device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v, int lane) {
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    unsigned n = __shfl_up(v, off);
-    if (lane >= off) v += n;
-  }
+// Inclusive prefix sum over the wave's 64 lanes with data-parallel-primitive moves: shifts within
+// rows of 16 lanes (lanes shifted in from outside a row read 0), then lane 15 of a row added to the
+// whole next row and lane 31 to the upper half of the wave. Every lane of the wave must be active.
+__device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v, int /*lane*/) {
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31
   return v;
 }
 
@@ -899,10 +903,10 @@ __global__ __launch_bounds__(256) void finalize_scatter_kernel(
 // Any window, TC blocks at a time: rows may hold repeated or descending columns. sCnt
 // ([TC * 16]) and sBm ([TC * WPT]) are the caller's LDS; sRow holds the window's 17 row pointers;
 // *sUnsorted must be 0 on entry. Every thread of the workgroup calls this.
-template <int W, int TB, int TC>
+template <int W, int TB>
 __device__ __forceinline__ void fill_window_generic(
     const int32_t* __restrict__ colIdx, const int32_t* __restrict__ edgeToColumn, int w, int base,
-    int nb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
+    int nb, const int TC, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
     int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
     unsigned long long* __restrict__ bitmap, unsigned* sCnt, unsigned long long* sBm,
     const int* sRow, unsigned* sWaveTot, unsigned* sUnsortedPtr) {
@@ -1068,8 +1072,8 @@ __device__ __forceinline__ void fill_window_generic(
         const bool inr = valid && (unsigned)t < (unsigned)nt;
         unsigned long long peers = __ballot(inr);
         if (peers == 0ull) continue;
-#pragma unroll
-        for (int b = 0; b < 9; b++) {
+        // lanes whose edges fall into the same block: agree on every bit of t (t < TC)
+        for (int b = 0; ((TC - 1) >> b) != 0; b++) {
           const unsigned long long bal = __ballot((t >> b) & 1);
           peers &= ((t >> b) & 1) ? bal : ~bal;
         }
@@ -1096,9 +1100,10 @@ template <int W, int TB, int TC, int TCG>
 __global__ __launch_bounds__(TB) void window_fill_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
     const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
-    long long nTcb, int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
-    int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
-    unsigned long long* __restrict__ bitmap, int minBlocks, int maxBlocks) {
+    const WsHeader* __restrict__ hdr, int32_t* __restrict__ tcblockRowid,
+    uint8_t* __restrict__ tcblocktileId, int32_t* __restrict__ tcblockOffset,
+    int32_t* __restrict__ sparseAToXidx, unsigned long long* __restrict__ bitmap, int minBlocks,
+    int maxBlocks) {
   constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
   constexpr int LOGW = (W == 16) ? 4 : 3;
   constexpr int FAST_BYTES = TC * (WPT * 8 + W * 4);
@@ -1115,8 +1120,11 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int w = blockIdx.x;
+  // launched right behind phase 1 (no host in between): a column index outside [0, N) left
+  // edgeToColumn unwritten, so nothing here may run
+  if (hdr && hdr->error) return;
   if (tid == 0) sUnsorted = 0u;
-  if (w == 0 && tid == 0) tcblockOffset[nTcb] = E;
+  if (w == 0 && tid == 0) tcblockOffset[rowWindowOffset[gridDim.x]] = E;
   const int base = rowWindowOffset[w];
   const int nb = rowWindowOffset[w + 1] - base;
   // a launch may be one of two that share the windows by length: [minBlocks, maxBlocks]
@@ -1249,9 +1257,436 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
     __syncthreads();
     unsigned* gCnt = reinterpret_cast<unsigned*>(sRaw);                                  // [TCG*16]
     unsigned long long* gBm = reinterpret_cast<unsigned long long*>(sRaw + TCG * 64);    // [TCG*WPT]
-    fill_window_generic<W, TB, TCG>(colIdx, edgeToColumn, w, base, nb, tcblockRowid,
-                                    tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, gCnt, gBm,
-                                    sRow, sWaveTot, &sUnsorted);
+    fill_window_generic<W, TB>(colIdx, edgeToColumn, w, base, nb, TCG, tcblockRowid,
+                               tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, gCnt, gBm, sRow,
+                               sWaveTot, &sUnsorted);
+  }
+}
+
+// ------------------------------------------------------------------ both phases, one call
+// Graphs of long windows whose column range fits one bitset (N <= kRangeMax) when the caller has
+// sized the block arrays by an upper bound instead of waiting for the count: the window's bitset
+// is built twice (window_count_kernel for the block counts, window_rank_fill_kernel after the
+// scan) and everything else happens while it sits in LDS, so edgeToColumn is written once and
+// never read back and the column ids are read from memory once (the second and third reads of a
+// window's 30 KB come from the L2).
+//
+// Neither kernel is bound by memory (on a 115 M-edge graph the vector ALUs are busy about half of
+// the time and HBM a quarter), so they are written for few instructions per edge: a window's edges are split into whole groups of four consecutive edges
+// from a 4-aligned index (no per-edge range checks, 16-byte loads and stores) and at most six
+// edges at the window's two ends, which single threads handle one by one.
+
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for the
+// wave's outstanding global loads and stores, which then overlap the next phase. For phases that
+// talk to each other through LDS and never through global memory.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Writes a TC block's tile ids (row * W + column of every set bit, rows top to bottom, columns
+// left to right) to dst[pos...]. words: the block's bitmap, 8x8 sub-blocks in column-major order.
+template <int W>
+__device__ __forceinline__ void walk_tile_ids(const unsigned long long (&words)[16 * W / 64],
+                                              uint8_t* __restrict__ dst, unsigned pos) {
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    unsigned rowBits = 0;  // W bits, column 0 in the most significant one
+#pragma unroll
+    for (int h = 0; h < W / 8; h++)
+      rowBits = (rowBits << 8) |
+                ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
+    while (rowBits) {
+      const int cl = __clz(rowBits) - (32 - W);
+      dst[pos++] = (uint8_t)(r * W + cl);
+      rowBits &= ~(1u << (W - 1 - cl));
+    }
+  }
+}
+
+// The window's edges [eS, eE) as whole 4-aligned groups [gA, gB) plus the edges in front of and
+// behind them (at most three each).
+struct EdgeSplit {
+  int gA, gB;      // whole groups: e0 = gA, gA + 4, ... < gB
+  int headEnd;     // loose edges [eS, headEnd) and [tailBegin, eE)
+  int tailBegin;
+};
+__device__ __forceinline__ EdgeSplit split_edges(int eS, int eE) {
+  EdgeSplit sp;
+  const int up = (eS + 3) & ~3, down = eE & ~3;
+  sp.headEnd = min(up, eE);
+  sp.tailBegin = max(down, sp.headEnd);
+  sp.gA = up;
+  sp.gB = max(down, up);
+  return sp;
+}
+// the i-th loose edge (i = 0..5), or -1
+__device__ __forceinline__ int loose_edge(const EdgeSplit& sp, int eS, int eE, int i) {
+  const int nHead = sp.headEnd - eS;
+  const int e = i < nHead ? eS + i : sp.tailBegin + (i - nHead);
+  return (i < 6 && e < eE) ? e : -1;
+}
+
+// Sets the bits of the window's column ids in `bits` (32-bit words). Returns false (for the
+// calling thread) when it met a column outside [0, N).
+template <int TB>
+__device__ __forceinline__ bool set_column_bits(const int32_t* __restrict__ colIdx, int eS, int eE,
+                                                const EdgeSplit& sp, unsigned N, uint32_t* bits) {
+  const int tid = threadIdx.x;
+  bool ok = true;
+  // two groups per thread and step, loads first
+  for (int e0 = sp.gA + 4 * tid; e0 < sp.gB; e0 += 8 * TB) {
+    const int4 a = *reinterpret_cast<const int4*>(colIdx + e0);
+    const bool two = e0 + 4 * TB < sp.gB;
+    int4 b = a;
+    if (two) b = *reinterpret_cast<const int4*>(colIdx + e0 + 4 * TB);
+    const unsigned c[8] = {(unsigned)a.x, (unsigned)a.y, (unsigned)a.z, (unsigned)a.w,
+                           (unsigned)b.x, (unsigned)b.y, (unsigned)b.z, (unsigned)b.w};
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      if (c[u] < N)
+        atomicOr(&bits[c[u] >> 5], 1u << (c[u] & 31));
+      else
+        ok = false;
+    }
+  }
+  const int e = loose_edge(sp, eS, eE, tid);
+  if (e >= 0) {
+    const unsigned c = (unsigned)colIdx[e];
+    if (c < N)
+      atomicOr(&bits[c >> 5], 1u << (c & 31));
+    else
+      ok = false;
+  }
+  return ok;
+}
+
+template <int W, int TB>
+__global__ __launch_bounds__(TB) void window_count_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int range,
+    int32_t* __restrict__ blockPartition, WsHeader* __restrict__ hdr) {
+  extern __shared__ __align__(16) uint32_t smem[];
+  uint32_t* bits = smem;  // range/32 words
+  __shared__ unsigned sWaveTot[TB / 64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int w = blockIdx.x;
+  const int eS = rowPtr[min(w * 16, N)], eE = rowPtr[min(w * 16 + 16, N)];
+  if (eE <= eS) {
+    if (tid == 0) blockPartition[w] = 0;
+    return;
+  }
+  const int nGroups = range >> 7;
+  for (int i = tid; i < nGroups; i += TB)
+    reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
+  lds_barrier();
+  const EdgeSplit sp = split_edges(eS, eE);
+  if (!set_column_bits<TB>(colIdx, eS, eE, sp, (unsigned)N, bits)) atomicOr(&hdr->error, 1);
+  lds_barrier();
+  unsigned cnt = 0;
+  for (int gi = tid; gi < nGroups; gi += TB) {
+    const uint4 v = reinterpret_cast<const uint4*>(bits)[gi];
+    cnt += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+  }
+  const unsigned incl = wave_inclusive_scan(cnt, lane);
+  if (lane == 63) sWaveTot[wave] = incl;
+  lds_barrier();
+  if (tid == 0) {
+    unsigned total = 0;
+#pragma unroll
+    for (int v = 0; v < TB / 64; v++) total += sWaveTot[v];
+    blockPartition[w] = (int)((total + W - 1) / W);
+  }
+}
+
+constexpr int kRankFillThreads = 768;
+// 64-bit bitset words per thread of window_rank_fill_kernel at the largest column range
+constexpr int kRankFillPerMax = (kRangeMax / 64 + kRankFillThreads - 1) / kRankFillThreads;
+
+// Dynamic LDS: bitset (range/64 64-bit words) | set bits before each word (range/64 32-bit words)
+// | chunkBytes of TC-block bitmaps. A window with a repeated or descending column is handed to
+// fill_window_generic once its edgeToColumn entries are written, with the whole of the dynamic LDS
+// as that routine's arrays.
+template <int W, int TB>
+__global__ __launch_bounds__(TB) __attribute__((amdgpu_waves_per_eu(6, 6)))
+void window_rank_fill_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
+    int range, int chunkBytes, const int32_t* __restrict__ rowWindowOffset,
+    const WsHeader* __restrict__ hdr, int32_t* edgeToColumn, int32_t* __restrict__ edgeToRow,
+    int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
+    int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
+    unsigned long long* __restrict__ bitmap) {
+  constexpr int WPT = 16 * W / 64;  // bitmap words per TC block
+  constexpr int LOGW = (W == 16) ? 4 : 3;
+  constexpr int NWAVE = TB / 64;
+  constexpr int PER = kRankFillPerMax;
+  static_assert(TB == kRankFillThreads, "PER is computed for this workgroup size");
+  extern __shared__ __align__(16) uint32_t smem[];
+  const int nW64 = range >> 6;  // even: range is a multiple of 128
+  unsigned long long* bits64 = reinterpret_cast<unsigned long long*>(smem);
+  uint32_t* bits = smem;
+  uint32_t* pref = smem + 2 * nW64;
+  const int bitsetWords = (3 * nW64 + 3) & ~3;  // 32-bit words of bitset + prefixes, 16-byte padded
+  unsigned long long* sBm = reinterpret_cast<unsigned long long*>(smem + bitsetWords);
+  const int TC = chunkBytes / (WPT * 8);
+  __shared__ int sRow[17];
+  __shared__ unsigned sWaveTot[NWAVE];
+  __shared__ unsigned sTot[PER * NWAVE];  // set bits per (round, wave), then their exclusive scan
+  __shared__ unsigned sUnsorted;          // bit r: row r's columns are not strictly ascending
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int w = blockIdx.x;
+  if (hdr->error) return;  // a column index outside [0, N): the caller gets the error, no output
+  if (w == 0 && tid == 0) tcblockOffset[rowWindowOffset[gridDim.x]] = E;
+  const int base = rowWindowOffset[w];
+  const int nb = rowWindowOffset[w + 1] - base;
+  const int r0 = w * 16;
+  if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
+  if (tid == 0) sUnsorted = 0u;
+  for (int i = tid; i < (nW64 >> 1); i += TB)
+    reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
+  lds_barrier();
+  const int eS = sRow[0], eE = sRow[16];
+  if (eE <= eS) return;
+  const EdgeSplit sp = split_edges(eS, eE);
+
+  // ---- the window's distinct columns as a bitset (validated by window_count_kernel)
+  set_column_bits<TB>(colIdx, eS, eE, sp, (unsigned)N, bits);
+  lds_barrier();
+
+  // ---- set bits before every 64-bit word; the compacted column ids, which are the set bits in
+  // ascending order. Thread t owns the words t, t + TB, ... (neighbouring lanes, neighbouring
+  // words): a wave-level scan per round, one scan of the (round, wave) totals by the first wave.
+  const int per = (nW64 + TB - 1) / TB;  // <= PER
+#pragma unroll
+  for (int k = 0; k < PER; k++) {
+    if (k < per) {
+      const int i = k * TB + tid;
+      const unsigned cnt = i < nW64 ? (unsigned)__popcll(bits64[i]) : 0u;
+      const unsigned incl = wave_inclusive_scan(cnt, lane);
+      if (i < nW64) pref[i] = incl - cnt;  // within the wave's 64 words for now
+      if (lane == 63) sTot[k * NWAVE + wave] = incl;
+    }
+  }
+  lds_barrier();
+  if (wave == 0) {
+    // exclusive scan of the per * NWAVE totals in (round, wave) order, two per lane
+    static_assert(PER * NWAVE <= 128, "two totals per lane");
+    const int n = per * NWAVE;
+    const unsigned a = (2 * lane < n) ? sTot[2 * lane] : 0u;
+    const unsigned b = (2 * lane + 1 < n) ? sTot[2 * lane + 1] : 0u;
+    const unsigned inc = wave_inclusive_scan(a + b, lane);
+    if (2 * lane < n) sTot[2 * lane] = inc - a - b;
+    if (2 * lane + 1 < n) sTot[2 * lane + 1] = inc - b;
+    if (lane == 63) sWaveTot[0] = inc;
+  }
+  lds_barrier();
+  const unsigned nCols = sWaveTot[0];
+  {
+    int32_t* idDst = sparseAToXidx + (int64_t)base * W;
+    char* idBytes = reinterpret_cast<char*>(idDst);
+    for (int k = 0; k < per; k++) {
+      const int i = k * TB + tid;
+      if (i < nW64) {
+        unsigned pos = sTot[k * NWAVE + wave] + pref[i];
+        pref[i] = pos;
+        // 32 bits at a time, with a 32-bit byte offset from the window's first id slot
+        const unsigned long long x = bits64[i];
+        unsigned off = pos * 4u;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          unsigned half = h ? (unsigned)(x >> 32) : (unsigned)x;
+          const int idBase = i * 64 + 32 * h;
+          while (half) {
+            *reinterpret_cast<int32_t*>(idBytes + off) = idBase + __builtin_ctz(half);
+            off += 4u;
+            half &= half - 1u;
+          }
+        }
+      }
+    }
+    // the slots that the last block leaves unused hold 0
+    for (int i = (int)nCols + tid; i < nb * W; i += TB) idDst[i] = 0;
+  }
+
+  // ---- ranks, rows and bitmaps. The first chunk of TC blocks also writes edgeToColumn /
+  // edgeToRow; a window with more blocks ranks its edges again per chunk (the bitset stays in
+  // LDS).
+  auto rank_of = [&](int col) -> int {
+    const unsigned wd = (unsigned)col >> 6;
+    const unsigned long long below = bits64[wd] & ((1ull << (col & 63)) - 1ull);
+    return (int)(pref[wd] + (unsigned)__popcll(below));
+  };
+  unsigned carry = (unsigned)eS;  // absolute edge position where the next TC block starts
+  unsigned* sBmWords = reinterpret_cast<unsigned*>(sBm);
+  const int stageBytes = ((bitsetWords * 4) / NWAVE) & ~15;
+  for (int tc0 = 0; tc0 < nb; tc0 += TC) {
+    const int nt = min(TC, nb - tc0);
+    const bool lastChunk = tc0 + TC >= nb;
+    const bool first = tc0 == 0;
+    lds_barrier();  // ranks are read after the prefixes are written (and the previous chunk is out)
+    for (int i = tid; i < nt * WPT; i += TB) sBm[i] = 0ull;
+    lds_barrier();
+    // one edge: rank, row, bit (the window's loose ends and groups that straddle rows)
+    auto one_edge = [&](int e, int col, int r) {
+      const int ec = rank_of(col);
+      if (first) {
+        edgeToColumn[e] = ec;
+        edgeToRow[e] = r0 + r;
+        if (e > sRow[r] && colIdx[e - 1] >= col) atomicOr(&sUnsorted, 1u << r);
+      }
+      const int t = (ec >> LOGW) - tc0;
+      if ((unsigned)t < (unsigned)nt) {
+        const int cl = ec & (W - 1);
+        const int sub = (cl >> 3) * (W / 8) + (r >> 3);
+        const int key = (t * WPT + sub) * 8 + 7 - (r & 7);
+        atomicOr(&sBmWords[key >> 2], (0x80u >> (cl & 7)) << (8 * (key & 3)));
+      }
+    };
+    // a whole group of four edges
+    auto group = [&](int e0, const int4& c4, int left) {
+      const int cols[4] = {c4.x, c4.y, c4.z, c4.w};
+      const int r = row_of_edge(sRow, e0);
+      if (e0 + 3 >= sRow[r + 1]) {  // the group straddles rows
+#pragma unroll
+        for (int u = 0; u < 4; u++) one_edge(e0 + u, cols[u], row_of_edge(sRow, e0 + u));
+        return;
+      }
+      int ecs[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) ecs[u] = rank_of(cols[u]);
+      if (first) {
+        *reinterpret_cast<int4*>(edgeToColumn + e0) = make_int4(ecs[0], ecs[1], ecs[2], ecs[3]);
+        *reinterpret_cast<int4*>(edgeToRow + e0) = make_int4(r0 + r, r0 + r, r0 + r, r0 + r);
+        const bool bad = (e0 > sRow[r] && left >= cols[0]) || cols[0] >= cols[1] ||
+                         cols[1] >= cols[2] || cols[2] >= cols[3];
+        if (bad) atomicOr(&sUnsorted, 1u << r);
+      }
+      // Bits of one row. A TC block's bitmap is WPT 64-bit words, one per 8x8 sub-block (column
+      // halves first); byte 7 - r%8 of a word is row r%8, MSB first. With rank = 16 t + cl (or
+      // 8 t + cl) the 64-bit word of (t, cl, r) is 2 (rank >> 3) + (r >> 3) for both widths, and
+      // the bit inside the row's byte is 0x80 >> (rank & 7). Consecutive edges of a row fall into
+      // the same byte up to eight at a time: OR the bits of equal bytes together, then one
+      // 32-bit LDS atomic per byte.
+      const int byte = 7 - (r & 7);
+      const int wordBias = (r >> 3) * 2 + (byte >> 2) - tc0 * (WPT * 2);  // in 32-bit words
+      const unsigned rowBit = 0x80u << (8 * (byte & 3));
+      int word[4];
+      unsigned m[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        word[u] = (ecs[u] >> 3) * 4 + wordBias;
+        m[u] = rowBit >> (ecs[u] & 7);
+        if ((unsigned)((ecs[u] >> LOGW) - tc0) >= (unsigned)nt) m[u] = 0u;
+      }
+#pragma unroll
+      for (int u = 1; u < 4; u++) {
+        if (word[u] == word[u - 1]) {
+          m[u] |= m[u - 1];
+          m[u - 1] = 0u;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (m[u]) atomicOr(&sBmWords[word[u]], m[u]);
+    };
+    // two groups per thread and step, loads first
+    for (int e0 = sp.gA + 4 * tid; e0 < sp.gB; e0 += 8 * TB) {
+      const int e1 = e0 + 4 * TB;
+      const bool two = e1 < sp.gB;
+      const int4 a = *reinterpret_cast<const int4*>(colIdx + e0);
+      int4 b = a;
+      if (two) b = *reinterpret_cast<const int4*>(colIdx + e1);
+      int leftA = -1, leftB = -1;
+      if (first) {
+        if (e0 > eS) leftA = colIdx[e0 - 1];
+        if (two) leftB = colIdx[e1 - 1];
+      }
+      group(e0, a, leftA);
+      if (two) group(e1, b, leftB);
+    }
+    {
+      const int e = loose_edge(sp, eS, eE, tid);
+      if (e >= 0) one_edge(e, colIdx[e], row_of_edge(sRow, e));
+    }
+    lds_barrier();
+    if (sUnsorted != 0u) break;  // known after the first pass over the window's edges
+    for (int tb = 0; tb < nt; tb += TB) {
+      const int t = tb + tid;
+      unsigned long long words[WPT];
+      unsigned nnz = 0;
+      if (t < nt) {
+#pragma unroll
+        for (int k = 0; k < WPT; k++) {
+          words[k] = sBm[t * WPT + k];
+          nnz += __popcll(words[k]);
+        }
+      }
+      const unsigned inc = wave_inclusive_scan(nnz, lane);
+      if (lane == 63) sWaveTot[wave] = inc;
+      lds_barrier();
+      unsigned waveOff = 0, tileTot = 0;
+#pragma unroll
+      for (int v = 0; v < NWAVE; v++) {
+        const unsigned x = sWaveTot[v];
+        if (v < wave) waveOff += x;
+        tileTot += x;
+      }
+      // tile ids: a block's set bits read row by row (src/utils.cu:213-223 walks the edges of a
+      // window with ascending rows in exactly that order). In the window's last chunk the bitset
+      // is no longer needed: each wave then collects the bytes of its 64 blocks in its slice of
+      // that LDS and writes them out as whole dwords.
+      const unsigned waveTot = __shfl(inc, 63);
+      const unsigned wavePos0 = carry + waveOff;
+      const unsigned a0 = wavePos0 & ~3u;
+      const bool staged = lastChunk && waveTot + 3u <= (unsigned)stageBytes;
+      uint8_t* stage = reinterpret_cast<uint8_t*>(smem) + wave * stageBytes;
+      if (t < nt) {
+        const int64_t gt = (int64_t)base + tc0 + t;
+        const unsigned pos = wavePos0 + inc - nnz;
+        tcblockOffset[gt] = (int)pos;
+        tcblockRowid[gt] = w;
+        // two calls, so that each store knows its address space (LDS or global)
+        if (staged)
+          walk_tile_ids<W>(words, stage, pos - a0);
+        else
+          walk_tile_ids<W>(words, tcblocktileId, pos);
+      }
+      if (staged && waveTot != 0u) {
+        wave_lds_sync();
+        const unsigned end = wavePos0 + waveTot;
+        const unsigned d0 = min((wavePos0 + 3u) & ~3u, end);  // first whole dword
+        const unsigned d1 = max(end & ~3u, d0);                // end of the whole dwords
+        for (unsigned i = wavePos0 + lane; i < d0; i += 64) tcblocktileId[i] = stage[i - a0];
+        for (unsigned i = d0 + 4u * lane; i < d1; i += 256u)
+          *reinterpret_cast<uint32_t*>(tcblocktileId + i) =
+              *reinterpret_cast<const uint32_t*>(stage + (i - a0));
+        for (unsigned i = d1 + lane; i < end; i += 64) tcblocktileId[i] = stage[i - a0];
+        wave_lds_sync();
+      }
+      carry += tileTot;
+      lds_barrier();
+    }
+    {
+      unsigned long long* bmDst = bitmap + ((int64_t)base + tc0) * WPT;
+      for (int i = tid; i < nt * WPT; i += TB) bmDst[i] = sBm[i];
+    }
+  }
+  if (sUnsorted != 0u) {
+    // repeated or descending columns somewhere in the window: the general way, from the
+    // edgeToColumn entries written above (visible to the whole workgroup after the barrier)
+    __syncthreads();
+    if (tid == 0) sUnsorted = 0u;
+    __syncthreads();
+    const int dynBytes = bitsetWords * 4 + chunkBytes;
+    const int tcg = dynBytes / (64 + WPT * 8);
+    unsigned* gCnt = reinterpret_cast<unsigned*>(smem);                                // [tcg*16]
+    unsigned long long* gBm = reinterpret_cast<unsigned long long*>(smem + tcg * 16);  // [tcg*WPT]
+    fill_window_generic<W, TB>(colIdx, edgeToColumn, w, base, nb, tcg, tcblockRowid,
+                               tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, gCnt, gBm, sRow,
+                               sWaveTot, &sUnsorted);
   }
 }
 
@@ -1287,6 +1722,45 @@ size_t preprocess_workspace_bytes(int N, int /*E*/) {
 
 namespace {
 
+// Scan of the block counts and the window order, after the kernels that write blockPartition.
+int enqueue_finalize(int N, int W, const int32_t* blockPartition, int32_t* rowWindowOffset,
+                     int32_t* sortedRowWindows, char* ws, hipStream_t stream) {
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
+  const size_t seg = align256((size_t)nRW * sizeof(int32_t));
+  int32_t* keysA = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes);
+  int32_t* keysB = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + seg);
+  int32_t* valsTmp = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + 2 * seg);
+  const int finWaves = finalize_waves(nRW);
+  if (finWaves == 0) {
+    hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
+                       nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
+    F3S_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
+  unsigned* waveSum = reinterpret_cast<unsigned*>(ws + kWsHeaderBytes + 3 * seg);
+  int* waveMax = reinterpret_cast<int*>(waveSum + finWaves);
+  unsigned* hist = waveSum + 2 * (size_t)finWaves;
+  const dim3 grid((unsigned)((finWaves + 3) / 4)), block(256);
+  hipLaunchKernelGGL(finalize_partials_kernel, grid, block, 0, stream, blockPartition, nRW,
+                     finWaves, waveSum, waveMax);
+  hipLaunchKernelGGL(finalize_scan_kernel, grid, block, 0, stream, blockPartition, nRW, finWaves,
+                     waveSum, waveMax, rowWindowOffset, hist, hdr);
+  // a window holds at most ceil(N / W) blocks: that bounds the passes that can be needed
+  int maxBits = 0;
+  while ((((int64_t)N + W - 1) / W >> maxBits) != 0) maxBits++;
+  const int maxPass = (maxBits + kFinDigitBits - 1) / kFinDigitBits;
+  for (int pass = 0; pass < (maxPass > 0 ? maxPass : 1); pass++) {
+    if (pass > 0)
+      hipLaunchKernelGGL(finalize_histogram_kernel, grid, block, 0, stream, nRW, finWaves, pass,
+                         keysA, keysB, hist, hdr);
+    hipLaunchKernelGGL(finalize_scatter_kernel, grid, block, 0, stream, blockPartition, nRW,
+                       finWaves, pass, sortedRowWindows, keysA, keysB, valsTmp, hist, hdr);
+  }
+  F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
 // Enqueues every kernel of phase 1 on `stream`; `ws` is device scratch of
 // preprocess_workspace_bytes(N, E) bytes whose header ends up holding the TC-block total and the
 // error flag.
@@ -1297,8 +1771,6 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
   const int nRW = (N + kWinRows - 1) / kWinRows;
   WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
   const size_t seg = align256((size_t)nRW * sizeof(int32_t));
-  int32_t* keysA = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes);
-  int32_t* keysB = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + seg);
   int32_t* valsTmp = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + 2 * seg);
 
   hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(1), 0, stream, hdr);
@@ -1365,34 +1837,7 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
 #undef F3S_RANK
     F3S_HIP_CHECK(hipGetLastError());
   }
-  const int finWaves = finalize_waves(nRW);
-  if (finWaves == 0) {
-    hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
-                       nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
-    F3S_HIP_CHECK(hipGetLastError());
-    return 0;
-  }
-  unsigned* waveSum = reinterpret_cast<unsigned*>(ws + kWsHeaderBytes + 3 * seg);
-  int* waveMax = reinterpret_cast<int*>(waveSum + finWaves);
-  unsigned* hist = waveSum + 2 * (size_t)finWaves;
-  const dim3 grid((unsigned)((finWaves + 3) / 4)), block(256);
-  hipLaunchKernelGGL(finalize_partials_kernel, grid, block, 0, stream, blockPartition, nRW,
-                     finWaves, waveSum, waveMax);
-  hipLaunchKernelGGL(finalize_scan_kernel, grid, block, 0, stream, blockPartition, nRW, finWaves,
-                     waveSum, waveMax, rowWindowOffset, hist, hdr);
-  // a window holds at most ceil(N / W) blocks: that bounds the passes that can be needed
-  int maxBits = 0;
-  while ((((int64_t)N + W - 1) / W >> maxBits) != 0) maxBits++;
-  const int maxPass = (maxBits + kFinDigitBits - 1) / kFinDigitBits;
-  for (int pass = 0; pass < (maxPass > 0 ? maxPass : 1); pass++) {
-    if (pass > 0)
-      hipLaunchKernelGGL(finalize_histogram_kernel, grid, block, 0, stream, nRW, finWaves, pass,
-                         keysA, keysB, hist, hdr);
-    hipLaunchKernelGGL(finalize_scatter_kernel, grid, block, 0, stream, blockPartition, nRW,
-                       finWaves, pass, sortedRowWindows, keysA, keysB, valsTmp, hist, hdr);
-  }
-  F3S_HIP_CHECK(hipGetLastError());
-  return 0;
+  return enqueue_finalize(N, W, blockPartition, rowWindowOffset, sortedRowWindows, ws, stream);
 }
 
 int check_count_args(const char* who, int N, int E, int H, int W) {
@@ -1485,20 +1930,16 @@ int launch_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx,
   return 0;
 }
 
-int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
-                           int W, const int32_t* edgeToColumn, const int32_t* rowWindowOffset,
-                           int64_t nTcb, int32_t* tcblockRowid, uint8_t* tcblocktileId,
-                           int32_t* tcblockOffset, int32_t* sparseAToXidx, uint64_t* bitmap,
-                           hipStream_t stream) {
-  if (H != 16 || (W != 16 && W != 8))
-    return fail(-2, "f3s_preprocess_fill: block %dx%d unsupported (16x16 or 16x8)", H, W);
+namespace {
+
+// Enqueues phase 2. `hdr` (may be null) is the header phase 1 left on the device: with it the
+// kernels do nothing after a column index error, so that phase 2 can follow phase 1 on the stream
+// without the host in between.
+int enqueue_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int W,
+                 const int32_t* edgeToColumn, const int32_t* rowWindowOffset, const WsHeader* hdr,
+                 int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                 int32_t* sparseAToXidx, uint64_t* bitmap, hipStream_t stream) {
   const int nRW = (N + kWinRows - 1) / kWinRows;
-  if (nRW == 0) {
-    hipLaunchKernelGGL(set_tail_kernel, dim3(1), dim3(1), 0, stream, tcblockOffset,
-                       (long long)nTcb, E);
-    F3S_HIP_CHECK(hipGetLastError());
-    return 0;
-  }
   auto bm = reinterpret_cast<unsigned long long*>(bitmap);
   // Windows with thousands of edges get eight waves and 512 TC blocks of LDS at a time. Graphs
   // of short windows get one wave per window and 128 blocks of LDS, so that a CU works on a
@@ -1506,8 +1947,8 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
   // more than 128 blocks are left to a second launch with four waves per window.
 #define F3S_FILL(WW, TBB, TCC, TCG, LO, HI)                                                    \
   hipLaunchKernelGGL((window_fill_kernel<WW, TBB, TCC, TCG>), dim3(nRW), dim3(TBB), 0, stream, \
-                     rowPtr, colIdx, N, E, edgeToColumn, rowWindowOffset, (long long)nTcb,     \
-                     tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx, bm, LO, HI)
+                     rowPtr, colIdx, N, E, edgeToColumn, rowWindowOffset, hdr, tcblockRowid,   \
+                     tcblocktileId, tcblockOffset, sparseAToXidx, bm, LO, HI)
   const bool big = (int64_t)E >= (int64_t)nRW * 2048;
   constexpr int kAll = 0x7FFFFFFF;
   if (W == 16) {
@@ -1529,6 +1970,107 @@ int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, 
   }
 #undef F3S_FILL
   F3S_HIP_CHECK(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+
+int launch_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,
+                           int W, const int32_t* edgeToColumn, const int32_t* rowWindowOffset,
+                           int64_t nTcb, int32_t* tcblockRowid, uint8_t* tcblocktileId,
+                           int32_t* tcblockOffset, int32_t* sparseAToXidx, uint64_t* bitmap,
+                           hipStream_t stream) {
+  if (H != 16 || (W != 16 && W != 8))
+    return fail(-2, "f3s_preprocess_fill: block %dx%d unsupported (16x16 or 16x8)", H, W);
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  if (nRW == 0) {
+    hipLaunchKernelGGL(set_tail_kernel, dim3(1), dim3(1), 0, stream, tcblockOffset,
+                       (long long)nTcb, E);
+    F3S_HIP_CHECK(hipGetLastError());
+    return 0;
+  }
+  return enqueue_fill(rowPtr, colIdx, N, E, W, edgeToColumn, rowWindowOffset, nullptr, tcblockRowid,
+                      tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, stream);
+}
+
+// ------------------------------------------------------- both phases behind one call
+int64_t preprocess_capacity(int N, int64_t E, int W) {
+  // a window of e edges names at most e distinct columns: ceil(e / W) <= e / W + 1 blocks
+  const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
+  return (E + W - 1) / W + nRW;
+}
+
+int launch_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                      int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                      int32_t* rowWindowOffset, int32_t* sortedRowWindows, int64_t capacity,
+                      int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                      int32_t* sparseAToXidx, uint64_t* bitmap, void* workspace, size_t wsBytes,
+                      int64_t* nTcbHost, hipStream_t stream) {
+  if (int rc = check_count_args("f3s_preprocess", N, E, H, W)) return rc;
+  if (wsBytes < preprocess_workspace_bytes(N, E))
+    return fail(-2, "f3s_preprocess: workspace %zu B < required %zu B", wsBytes,
+                preprocess_workspace_bytes(N, E));
+  if (capacity < preprocess_capacity(N, E, W))
+    return fail(-2, "f3s_preprocess: block arrays sized for %lld TC blocks, the bound for this "
+                    "graph is %lld (f3s_preprocess_capacity)",
+                (long long)capacity, (long long)preprocess_capacity(N, E, W));
+  char* ws = static_cast<char*>(workspace);
+  WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
+  const int nRW = (N + kWinRows - 1) / kWinRows;
+  const bool aligned16 =
+      ((reinterpret_cast<uintptr_t>(colIdx) | reinterpret_cast<uintptr_t>(edgeToColumn) |
+        reinterpret_cast<uintptr_t>(edgeToRow) | reinterpret_cast<uintptr_t>(sparseAToXidx) |
+        reinterpret_cast<uintptr_t>(tcblocktileId)) & 15u) == 0;
+  // long windows, one bitset pass: the kernels that keep a window's bitset in LDS for both phases
+  const bool fused = nRW > 0 && (int64_t)E >= (int64_t)nRW * 2048 && N <= kRangeMax && aligned16;
+  if (fused) {
+    const int range = ((N + 127) / 128) * 128;
+    const int bitsetBytes = ((3 * (range / 64) + 3) & ~3) * 4;  // bitset + per-word prefixes
+    // two workgroups of twelve waves per CU (registers allow no more): half of the CU's LDS each
+    int chunkBytes = (160 * 1024) / 2 - 1024 - bitsetBytes;
+    chunkBytes &= ~255;
+    const size_t ldsCount = (size_t)(range / 32) * 4;
+    const size_t ldsFill = (size_t)bitsetBytes + chunkBytes;
+    hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(1), 0, stream, hdr);
+#define F3S_ONECALL(WW)                                                                        \
+  do {                                                                                         \
+    if (ldsFill > 64 * 1024)                                                                   \
+      F3S_HIP_CHECK(hipFuncSetAttribute(                                                       \
+          reinterpret_cast<const void*>(&window_rank_fill_kernel<WW, kRankFillThreads>),                    \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsFill));                          \
+    hipLaunchKernelGGL((window_count_kernel<WW, 512>), dim3(nRW), dim3(512), ldsCount, stream, \
+                       rowPtr, colIdx, N, range, blockPartition, hdr);                      \
+    F3S_HIP_CHECK(hipGetLastError());                                                          \
+    if (int rc = enqueue_finalize(N, W, blockPartition, rowWindowOffset, sortedRowWindows, ws, \
+                                  stream))                                                     \
+      return rc;                                                                               \
+    hipLaunchKernelGGL((window_rank_fill_kernel<WW, kRankFillThreads>), dim3(nRW),            \
+                       dim3(kRankFillThreads), ldsFill,                                          \
+                       stream, rowPtr, colIdx, N, E, range, chunkBytes, rowWindowOffset, hdr,  \
+                       edgeToColumn, edgeToRow, tcblockRowid, tcblocktileId, tcblockOffset,    \
+                       sparseAToXidx, reinterpret_cast<unsigned long long*>(bitmap));          \
+    F3S_HIP_CHECK(hipGetLastError());                                                          \
+  } while (0)
+    if (W == 16) F3S_ONECALL(16); else F3S_ONECALL(8);
+#undef F3S_ONECALL
+  } else {
+    if (int rc = enqueue_count(rowPtr, colIdx, N, E, W, blockPartition, edgeToColumn, edgeToRow,
+                               rowWindowOffset, sortedRowWindows, ws, stream))
+      return rc;
+    if (nRW == 0) {
+      hipLaunchKernelGGL(set_tail_kernel, dim3(1), dim3(1), 0, stream, tcblockOffset, 0ll, E);
+      F3S_HIP_CHECK(hipGetLastError());
+    } else if (int rc = enqueue_fill(rowPtr, colIdx, N, E, W, edgeToColumn, rowWindowOffset, hdr,
+                                     tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx,
+                                     bitmap, stream)) {
+      return rc;
+    }
+  }
+  WsHeader host;
+  F3S_HIP_CHECK(hipMemcpyAsync(&host, ws, sizeof(WsHeader), hipMemcpyDeviceToHost, stream));
+  F3S_HIP_CHECK(hipStreamSynchronize(stream));
+  if (host.error) return fail(-4, "f3s_preprocess: column index outside [0, %d)", N);
+  *nTcbHost = host.nTcb;
   return 0;
 }
 

@@ -11,6 +11,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <fstream>
 #include <iomanip>
 #include <map>
@@ -37,6 +38,13 @@ void* current_stream() { return static_cast<void*>(at::hip::getCurrentHIPStream(
 bool verbose() {
   const char* v = std::getenv("F3S_VERBOSE");
   return v && v[0] != '\0' && v[0] != '0';
+}
+
+// F3S_PREPROCESS=two_phase: count, exact allocations, fill, as the reference does; default: one
+// call with the block arrays allocated for a bound on the block total (read per call)
+bool two_phase() {
+  const char* v = std::getenv("F3S_PREPROCESS");
+  return v && std::strcmp(v, "two_phase") == 0;
 }
 
 // F3S.preprocess_gpu (src/F3S.cpp:40-87). The three caller tensors are filled in place as in
@@ -75,27 +83,56 @@ preprocess_gpu(torch::Tensor edgeList, torch::Tensor nodePointer, int num_nodes,
   const size_t wsBytes = f3s_preprocess_workspace_bytes(num_nodes, (int)E);
   auto workspace = torch::empty({(int64_t)wsBytes}, i32.dtype(torch::kUInt8));
   int64_t nTcb = 0;
-  check_status(
-      f3s_preprocess_count(nodePointer.data_ptr<int>(), edgeList.data_ptr<int>(), num_nodes,
-                           (int)E, blockSize_h, blockSize_w, blockPartition.data_ptr<int>(),
-                           edgeToColumn.data_ptr<int>(), edgeToRow.data_ptr<int>(),
-                           rowWindowOffset.data_ptr<int>(), sortedRowWindows.data_ptr<int>(),
-                           workspace.data_ptr(), wsBytes, &nTcb, current_stream()),
-      "f3s_preprocess_count");
-  auto tcblockRowid = torch::empty({nTcb}, i32);
   auto tcblocktileId = torch::empty({E}, i32.dtype(torch::kUInt8));
-  auto tcblockOffset = torch::empty({nTcb + 1}, i32);
-  auto sparseAToXidx = torch::empty({nTcb * blockSize_w}, i32);
-  auto tcbBitMap =
-      torch::empty({nTcb * blockSize_h * blockSize_w / 64}, i32.dtype(torch::kUInt64));
-  check_status(
-      f3s_preprocess_fill(nodePointer.data_ptr<int>(), edgeList.data_ptr<int>(), num_nodes, (int)E,
-                          blockSize_h, blockSize_w, edgeToColumn.data_ptr<int>(),
-                          rowWindowOffset.data_ptr<int>(), nTcb, tcblockRowid.data_ptr<int>(),
-                          tcblocktileId.data_ptr<uint8_t>(), tcblockOffset.data_ptr<int>(),
-                          sparseAToXidx.data_ptr<int>(),
-                          reinterpret_cast<uint64_t*>(tcbBitMap.data_ptr()), current_stream()),
-      "f3s_preprocess_fill");
+  torch::Tensor tcblockRowid, tcblockOffset, sparseAToXidx, tcbBitMap;
+  const int64_t bmWords = (int64_t)blockSize_h * blockSize_w / 64;
+  if (two_phase()) {
+    // the reference's sequence: count, allocate exactly, fill
+    check_status(
+        f3s_preprocess_count(nodePointer.data_ptr<int>(), edgeList.data_ptr<int>(), num_nodes,
+                             (int)E, blockSize_h, blockSize_w, blockPartition.data_ptr<int>(),
+                             edgeToColumn.data_ptr<int>(), edgeToRow.data_ptr<int>(),
+                             rowWindowOffset.data_ptr<int>(), sortedRowWindows.data_ptr<int>(),
+                             workspace.data_ptr(), wsBytes, &nTcb, current_stream()),
+        "f3s_preprocess_count");
+    tcblockRowid = torch::empty({nTcb}, i32);
+    tcblockOffset = torch::empty({nTcb + 1}, i32);
+    sparseAToXidx = torch::empty({nTcb * blockSize_w}, i32);
+    tcbBitMap = torch::empty({nTcb * bmWords}, i32.dtype(torch::kUInt64));
+    check_status(
+        f3s_preprocess_fill(nodePointer.data_ptr<int>(), edgeList.data_ptr<int>(), num_nodes,
+                            (int)E, blockSize_h, blockSize_w, edgeToColumn.data_ptr<int>(),
+                            rowWindowOffset.data_ptr<int>(), nTcb, tcblockRowid.data_ptr<int>(),
+                            tcblocktileId.data_ptr<uint8_t>(), tcblockOffset.data_ptr<int>(),
+                            sparseAToXidx.data_ptr<int>(),
+                            reinterpret_cast<uint64_t*>(tcbBitMap.data_ptr()), current_stream()),
+        "f3s_preprocess_fill");
+  } else {
+    // one call: the block arrays are allocated for the bound on the block total and returned as
+    // views of their first nTcb entries, so the host waits for the device once, at the end
+    TORCH_CHECK(blockSize_h == 16 && (blockSize_w == 16 || blockSize_w == 8),
+                "preprocess_gpu: block ", blockSize_h, "x", blockSize_w,
+                " unsupported (16x16 or 16x8)");
+    const int64_t cap = f3s_preprocess_capacity(num_nodes, E, blockSize_w);
+    tcblockRowid = torch::empty({cap}, i32);
+    tcblockOffset = torch::empty({cap + 1}, i32);
+    sparseAToXidx = torch::empty({cap * blockSize_w}, i32);
+    tcbBitMap = torch::empty({cap * bmWords}, i32.dtype(torch::kUInt64));
+    check_status(
+        f3s_preprocess(nodePointer.data_ptr<int>(), edgeList.data_ptr<int>(), num_nodes, (int)E,
+                       blockSize_h, blockSize_w, blockPartition.data_ptr<int>(),
+                       edgeToColumn.data_ptr<int>(), edgeToRow.data_ptr<int>(),
+                       rowWindowOffset.data_ptr<int>(), sortedRowWindows.data_ptr<int>(), cap,
+                       tcblockRowid.data_ptr<int>(), tcblocktileId.data_ptr<uint8_t>(),
+                       tcblockOffset.data_ptr<int>(), sparseAToXidx.data_ptr<int>(),
+                       reinterpret_cast<uint64_t*>(tcbBitMap.data_ptr()), workspace.data_ptr(),
+                       wsBytes, &nTcb, current_stream()),
+        "f3s_preprocess");
+    tcblockRowid = tcblockRowid.narrow(0, 0, nTcb);
+    tcblockOffset = tcblockOffset.narrow(0, 0, nTcb + 1);
+    sparseAToXidx = sparseAToXidx.narrow(0, 0, nTcb * blockSize_w);
+    tcbBitMap = tcbBitMap.narrow(0, 0, nTcb * bmWords);
+  }
   if (verbose()) {
     TORCH_CHECK(hipStreamSynchronize(at::hip::getCurrentHIPStream().stream()) == hipSuccess);
     std::chrono::duration<double> dt = std::chrono::high_resolution_clock::now() - start;

@@ -107,6 +107,35 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
                         int32_t* sparseAToXidx, uint64_t* tcbBitMap, void* stream);
 
 /*
+ * All of F3S.preprocess_gpu (src/F3S.cpp:40-87) behind one call, for callers that size the
+ * nTCB-long outputs by an upper bound instead of waiting for the count: both phases are enqueued
+ * back to back and the host reads the block total once, at the end. The reference allocates its
+ * block arrays between the phases (src/F3S.cpp:62-70 around the copy at src/utils.cu:307-309);
+ * a caller of this entry allocates them for f3s_preprocess_capacity(N, E, W) blocks beforehand
+ * and uses the first nTCB entries.
+ *
+ *   capacity       TC blocks the five block arrays below have room for; at least
+ *                  f3s_preprocess_capacity(N, E, W) = ceil(E / W) + ceil(N / 16), which bounds
+ *                  the total of any graph with these sizes
+ *   tcblockRowid [capacity], tcblocktileId [E], tcblockOffset [capacity+1],
+ *   sparseAToXidx [capacity*W], tcbBitMap [capacity*H*W/64]
+ *                  out: entries of the first nTCB blocks as f3s_preprocess_fill writes them
+ *                  (tcblockOffset: nTCB + 1 entries); the rest is left untouched
+ *   every other argument as in f3s_preprocess_count
+ * On graphs of long windows whose column range fits one LDS bitset (E >= 128 N, N <= 393 216)
+ * a window's ranking bitset stays in LDS for both phases, so edgeToColumn is written once and
+ * not read back. Synchronises `stream` before returning. Returns 0 or a negative status; after a
+ * column index outside [0, N) (-4) the outputs are undefined.
+ */
+int64_t f3s_preprocess_capacity(int N, int64_t E, int W);
+int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
+                   int32_t* blockPartition, int32_t* edgeToColumn, int32_t* edgeToRow,
+                   int32_t* rowWindowOffset, int32_t* sortedRowWindows, int64_t capacity,
+                   int32_t* tcblockRowid, uint8_t* tcblocktileId, int32_t* tcblockOffset,
+                   int32_t* sparseAToXidx, uint64_t* tcbBitMap, void* workspace, size_t ws_bytes,
+                   int64_t* nTCB_host, void* stream);
+
+/*
  * Fused SDDMM -> softmax -> SpMM over 16x16 TC blocks. Replaces f3sCuda1tb1rw,
  * f3sCuda1tb1rwScheduled (src/F3S_kernel.cu:393-458, 581-671) and the kernels they launch
  * (f3sKernel1tb1rw :997-1175, f3sKernel1tb1rwScheduled :1999-2182,

@@ -27,12 +27,20 @@ def to_host(res):
 
 
 def run_gpu(rowPtr, colIdx, N, W=16):
+    """Both entry styles: one call with bounded allocations (returned), and count / allocate /
+    fill, which must agree with it bit for bit."""
     from fused3s_amd import capi
     rp = torch.as_tensor(np.asarray(rowPtr, np.int32)).cuda()
     ci = torch.as_tensor(np.asarray(colIdx, np.int32)).cuda()
-    res = capi.preprocess(rp, ci, N, 16, W)
+    res = to_host(capi.preprocess(rp, ci, N, 16, W))
+    two = to_host(capi.preprocess(rp, ci, N, 16, W, two_phase=True))
     torch.cuda.synchronize()
-    return to_host(res)
+    for k, v in res.items():
+        if isinstance(v, np.ndarray):
+            assert v.shape == two[k].shape and np.array_equal(v, two[k]), k
+        else:
+            assert v == two[k], k
+    return res
 
 
 @pytest.mark.parametrize("case", KAT, ids=[c["name"] for c in KAT])
@@ -61,6 +69,75 @@ def test_random_graphs_bit_exact(oracle_mod, W, seed, N, deg, dup, unsorted, emp
     rowPtr, colIdx = random_csr(rng, N, deg, dup=dup, unsorted=unsorted, empty_frac=empty, hub=hub)
     got = run_gpu(rowPtr, colIdx, N, W)
     want = oracle_mod.preprocess(rowPtr, colIdx, N, 16, W)
+    compare_preprocess(got, want)
+
+
+def long_window_graph(rng, N, deg, messy_every=0, empty_every=0, hub_rows=0, hub_deg=0):
+    """Sorted duplicate-free rows of about `deg` entries; every messy_every-th row shuffled with a
+    third of its entries repeated; every empty_every-th row empty; the first hub_rows rows with
+    hub_deg entries."""
+    rows = []
+    for r in range(N):
+        if empty_every and r % empty_every == 3:
+            rows.append(np.zeros(0, np.int32))
+            continue
+        d = hub_deg if r < hub_rows else int(rng.poisson(deg))
+        cols = np.unique(rng.integers(0, N, size=d))
+        if messy_every and r % messy_every == 5:
+            cols = np.concatenate([cols, cols[: max(1, len(cols) // 3)]])
+            rng.shuffle(cols)
+        rows.append(cols.astype(np.int32))
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum([len(c) for c in rows])
+    return rowPtr, np.concatenate(rows).astype(np.int32)
+
+
+@pytest.mark.parametrize("W", [16, 8])
+@pytest.mark.parametrize("seed,N,deg,messy,empty", [
+    (0, 1000, 300, 0, 0),       # every window ascending
+    (1, 3001, 220, 40, 7),      # a messy row in some windows, empty rows, N % 16 != 0
+    (2, 777, 400, 1, 0),        # every row shuffled with repeats
+    (3, 20000, 150, 300, 50),
+])
+def test_long_windows_one_bitset_pass(oracle_mod, W, seed, N, deg, messy, empty):
+    """Graphs with >= 2048 edges per window and N <= 393216: the one-call entry keeps each
+    window's ranking bitset in LDS for both phases."""
+    print("case long windows seed=%d N=%d W=%d" % (seed, N, W), flush=True)
+    rng = np.random.default_rng(100 + seed)
+    rowPtr, colIdx = long_window_graph(rng, N, deg, messy, empty)
+    assert rowPtr[-1] >= ((N + 15) // 16) * 2048
+    got = run_gpu(rowPtr, colIdx, N, W)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N, 16, W)
+    compare_preprocess(got, want)
+
+
+@pytest.mark.parametrize("W", [16, 8])
+def test_long_windows_with_a_window_of_several_lds_chunks(oracle_mod, W):
+    """As above with one window of ~55 000 distinct columns (more TC blocks than the bitmaps'
+    share of LDS holds at once) and, with `messy`, the same window on the general path."""
+    print("case long windows, heavy window W=%d" % W, flush=True)
+    for messy in (0, 9):
+        rng = np.random.default_rng(7 + messy)
+        N = 100000
+        rowPtr, colIdx = long_window_graph(rng, N, 132, messy_every=messy, hub_rows=16,
+                                           hub_deg=5000)
+        assert rowPtr[-1] >= ((N + 15) // 16) * 2048
+        got = run_gpu(rowPtr, colIdx, N, W)
+        want = oracle_mod.preprocess(rowPtr, colIdx, N, 16, W)
+        assert want["blockPartition"][0] > (3000 if W == 16 else 6000)
+        compare_preprocess(got, want)
+
+
+def test_long_windows_quarter_scale_benchmark_graph(oracle_mod):
+    """The 233k-node benchmark graph at 0.3 of its size (same mean degree): large enough that the
+    waves collect their tile ids in LDS and write them as dwords."""
+    print("case cfg3 at scale 0.3", flush=True)
+    from fused3s_amd import synth
+    rp, ci = synth.make_graph("cfg3_chunglu_233k", scale=0.3, device="cuda")
+    rowPtr, colIdx = rp.cpu().numpy(), ci.cpu().numpy()
+    N = len(rowPtr) - 1
+    got = run_gpu(rowPtr, colIdx, N)
+    want = oracle_mod.preprocess(rowPtr, colIdx, N)
     compare_preprocess(got, want)
 
 
@@ -154,6 +231,15 @@ def test_out_of_range_column_is_an_error():
     ci = torch.tensor([0, 7], dtype=torch.int32).cuda()
     with pytest.raises(RuntimeError, match="column index"):
         capi.preprocess(rp, ci, 2)
+    with pytest.raises(RuntimeError, match="column index"):
+        capi.preprocess(rp, ci, 2, two_phase=True)
+    # long windows (the kernels that do both phases at once): 64 rows of 2100 entries, one bad
+    N = 64
+    rowPtr = torch.arange(N + 1, dtype=torch.int32) * 2100
+    cols = (torch.arange(N * 2100, dtype=torch.int32) % N)
+    cols[70000] = N
+    with pytest.raises(RuntimeError, match="column index"):
+        capi.preprocess(rowPtr.cuda(), cols.cuda(), N)
 
 
 @pytest.mark.parametrize("name,scale", [("cfg1_gnm_2708", 1.0), ("cfg2_rmat_169k", 1.0),
