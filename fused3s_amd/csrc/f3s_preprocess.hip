@@ -549,14 +549,22 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
 
 // ------------------------------------------------- scan + window ordering
 constexpr int kFinBlock = 1024;
+// windows the single-workgroup kernel takes: a window id fits kFinIdBits bits and a block count
+// (at most 16 * kFinSingleMax / 8 + 1) the rest of a 32-bit word
+constexpr int kFinSingleMax = 16384;
+constexpr int kFinIdBits = 14;
 
 __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     const int32_t* __restrict__ blockPartition, int nRW, int32_t* __restrict__ rowWindowOffset,
-    int32_t* __restrict__ sortedRowWindows, int32_t* __restrict__ keysA,
-    int32_t* __restrict__ keysB, int32_t* __restrict__ valsTmp, WsHeader* __restrict__ hdr) {
+    int32_t* __restrict__ sortedRowWindows, WsHeader* __restrict__ hdr) {
   // One workgroup; every wave owns a contiguous chunk of the windows and walks it on its own
   // (wave-level scans and ballots only), so a pass over the array costs a handful of block
-  // barriers instead of several per 1024 elements.
+  // barriers instead of several per 1024 elements. The sort's two buffers are in LDS
+  // (2 * kFinSingleMax words of dynamic LDS): a (key, window) pair is one word, key above
+  // kFinIdBits bits of window id.
+  extern __shared__ __align__(16) uint32_t finLds[];
+  uint32_t* bufA = finLds;
+  uint32_t* bufB = finLds + kFinSingleMax;
   constexpr int NW = kFinBlock / 64;
   __shared__ unsigned sWaveSum[NW];
   __shared__ int sWaveMax[NW];
@@ -623,12 +631,10 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   }
   const unsigned long long ltMask = (1ull << lane) - 1ull;
   for (int pass = 0; pass < nPass; pass++) {
-    const int shift = pass * DB;
-    const bool toOut = ((nPass - 1 - pass) & 1) == 0;
-    int32_t* kDst = toOut ? keysA : keysB;
-    int32_t* vDst = toOut ? sortedRowWindows : valsTmp;
-    const int32_t* kSrc = toOut ? keysB : keysA;
-    const int32_t* vSrc = toOut ? valsTmp : sortedRowWindows;
+    const int shift = kFinIdBits + pass * DB;
+    const bool last = pass == nPass - 1;
+    uint32_t* dst = (pass & 1) ? bufB : bufA;
+    const uint32_t* src = (pass & 1) ? bufA : bufB;
     __syncthreads();  // the previous pass's writes are visible, its use of sCnt is over
     sCnt[wave][lane] = 0;
     // peers = lanes of this 64-element group with the same digit (one ballot per digit bit)
@@ -641,18 +647,19 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
       }
       return peers;
     };
-    auto load_key = [&](int i) {
-      return (i < cEnd) ? ((pass == 0) ? (maxC - blockPartition[i]) : kSrc[i]) : 0;
+    auto load_key = [&](int i) -> unsigned {
+      if (i >= cEnd) return 0u;
+      return pass == 0 ? ((unsigned)(maxC - blockPartition[i]) << kFinIdBits) | (unsigned)i
+                       : src[i];
     };
-    auto load_val = [&](int i) { return (i < cEnd) ? ((pass == 0) ? i : vSrc[i]) : 0; };
     // histogram of the wave's chunk (the next group's keys are in flight during this one's)
-    int keyNext = load_key(cBegin + lane);
+    unsigned keyNext = load_key(cBegin + lane);
     for (int base = cBegin; base < cEnd; base += 64) {
       const int i = base + lane;
       const bool valid = i < cEnd;
-      const int key = keyNext;
+      const unsigned key = keyNext;
       keyNext = load_key(i + 64);
-      const int dgt = (key >> shift) & (NB - 1);
+      const int dgt = (int)(key >> shift) & (NB - 1);
       const unsigned long long peers = digit_peers(valid, dgt);
       if (valid && (peers & ltMask) == 0ull) sCnt[wave][dgt] += __popcll(peers);
     }
@@ -670,19 +677,19 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     sCnt[wave][lane] = start;
     // scatter, in order
     keyNext = load_key(cBegin + lane);
-    int valNext = load_val(cBegin + lane);
     for (int base = cBegin; base < cEnd; base += 64) {
       const int i = base + lane;
       const bool valid = i < cEnd;
-      const int key = keyNext, val = valNext;
+      const unsigned key = keyNext;
       keyNext = load_key(i + 64);
-      valNext = load_val(i + 64);
-      const int dgt = (key >> shift) & (NB - 1);
+      const int dgt = (int)(key >> shift) & (NB - 1);
       const unsigned long long peers = digit_peers(valid, dgt);
       if (valid) {
         const unsigned pos = sCnt[wave][dgt] + __popcll(peers & ltMask);
-        kDst[pos] = key;
-        vDst[pos] = val;
+        if (last)
+          sortedRowWindows[pos] = (int)(key & ((1u << kFinIdBits) - 1u));
+        else
+          dst[pos] = key;
       }
       // the last peer moves the digit's running position (the wave's LDS accesses stay in order)
       if (valid && (peers >> lane) == 1ull) sCnt[wave][dgt] += __popcll(peers);
@@ -1327,26 +1334,31 @@ __device__ __forceinline__ int loose_edge(const EdgeSplit& sp, int eS, int eE, i
 }
 
 // Sets the bits of the window's column ids in `bits` (32-bit words). Returns false (for the
-// calling thread) when it met a column outside [0, N).
-template <int TB>
+// calling thread) when it met a column outside [0, N). U groups per thread and step, loads first.
+template <int TB, int U>
 __device__ __forceinline__ bool set_column_bits(const int32_t* __restrict__ colIdx, int eS, int eE,
                                                 const EdgeSplit& sp, unsigned N, uint32_t* bits) {
   const int tid = threadIdx.x;
   bool ok = true;
-  // two groups per thread and step, loads first
-  for (int e0 = sp.gA + 4 * tid; e0 < sp.gB; e0 += 8 * TB) {
-    const int4 a = *reinterpret_cast<const int4*>(colIdx + e0);
-    const bool two = e0 + 4 * TB < sp.gB;
-    int4 b = a;
-    if (two) b = *reinterpret_cast<const int4*>(colIdx + e0 + 4 * TB);
-    const unsigned c[8] = {(unsigned)a.x, (unsigned)a.y, (unsigned)a.z, (unsigned)a.w,
-                           (unsigned)b.x, (unsigned)b.y, (unsigned)b.z, (unsigned)b.w};
+  for (int e0 = sp.gA + 4 * tid; e0 < sp.gB; e0 += 4 * U * TB) {
+    int4 c[U];
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      if (c[u] < N)
-        atomicOr(&bits[c[u] >> 5], 1u << (c[u] & 31));
-      else
-        ok = false;
+    for (int g = 0; g < U; g++) {
+      // a group past the end repeats the first one (its bits are set already)
+      const int e = e0 + 4 * g * TB < sp.gB ? e0 + 4 * g * TB : e0;
+      c[g] = *reinterpret_cast<const int4*>(colIdx + e);
+    }
+#pragma unroll
+    for (int g = 0; g < U; g++) {
+      const unsigned col[4] = {(unsigned)c[g].x, (unsigned)c[g].y, (unsigned)c[g].z,
+                               (unsigned)c[g].w};
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        if (col[u] < N)
+          atomicOr(&bits[col[u] >> 5], 1u << (col[u] & 31));
+        else
+          ok = false;
+      }
     }
   }
   const int e = loose_edge(sp, eS, eE, tid);
@@ -1381,7 +1393,7 @@ __global__ __launch_bounds__(TB) void window_count_kernel(
     reinterpret_cast<uint4*>(bits)[i] = make_uint4(0, 0, 0, 0);
   lds_barrier();
   const EdgeSplit sp = split_edges(eS, eE);
-  if (!set_column_bits<TB>(colIdx, eS, eE, sp, (unsigned)N, bits)) atomicOr(&hdr->error, 1);
+  if (!set_column_bits<TB, 4>(colIdx, eS, eE, sp, (unsigned)N, bits)) atomicOr(&hdr->error, 1);
   lds_barrier();
   unsigned cnt = 0;
   for (int gi = tid; gi < nGroups; gi += TB) {
@@ -1453,7 +1465,7 @@ void window_rank_fill_kernel(
   const EdgeSplit sp = split_edges(eS, eE);
 
   // ---- the window's distinct columns as a bitset (validated by window_count_kernel)
-  set_column_bits<TB>(colIdx, eS, eE, sp, (unsigned)N, bits);
+  set_column_bits<TB, 2>(colIdx, eS, eE, sp, (unsigned)N, bits);
   lds_barrier();
 
   // ---- set bits before every 64-bit word; the compacted column ids, which are the set bits in
@@ -1709,7 +1721,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // waves of the multi-workgroup finalize (0: the single-workgroup kernel is used)
 int finalize_waves(int nRW) {
-  if (nRW <= 16384) return 0;
+  if (nRW <= kFinSingleMax) return 0;
   const int w = (nRW + 511) / 512;
   return w < 4096 ? w : 4096;
 }
@@ -1733,8 +1745,11 @@ int enqueue_finalize(int N, int W, const int32_t* blockPartition, int32_t* rowWi
   int32_t* valsTmp = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + 2 * seg);
   const int finWaves = finalize_waves(nRW);
   if (finWaves == 0) {
-    hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), 0, stream, blockPartition,
-                       nRW, rowWindowOffset, sortedRowWindows, keysA, keysB, valsTmp, hdr);
+    constexpr int ldsBytes = 2 * kFinSingleMax * (int)sizeof(uint32_t);
+    F3S_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&finalize_count_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes));
+    hipLaunchKernelGGL(finalize_count_kernel, dim3(1), dim3(kFinBlock), ldsBytes, stream,
+                       blockPartition, nRW, rowWindowOffset, sortedRowWindows, hdr);
     F3S_HIP_CHECK(hipGetLastError());
     return 0;
   }
