@@ -20,6 +20,10 @@
 //                        scan of the per-window block counts (src/utils.cu:293-300) and a stable
 //                        LSD radix sort of the windows by descending block count
 //                        (src/utils.cu:400-436), ranks from wave ballots.
+//   window_count_kernel, window_rank_fill_kernel
+//                        graphs of long windows through the one-call entry: block counts, then
+//                        ranks, rows, ids, bitmaps and tile ids of a window while its bitset sits
+//                        in LDS.
 //   window_fill_kernel   one workgroup (or one wave, on graphs of short windows) per window:
 //                        bitmaps and per-(row, block) edge counts are accumulated in LDS, a scan
 //                        yields the per-block offsets, and the tile ids are written per block
