@@ -33,6 +33,10 @@ if ROOT not in sys.path:
 
 PEAK_MFMA_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16
 PEAK_HBM_GBPS = 8000.0
+# what the 256 vector L1s can hand to their CUs: 64 bytes per clock each at the 2.4 GHz peak engine
+# clock. Every K/V row of every TC block passes through them, so this bounds the gather whatever
+# the caches do (an attention call cannot be faster than B_gather over this).
+PEAK_L1_GBPS = 256 * 64 * 2.4
 
 
 def log(*a):
@@ -278,6 +282,7 @@ def run_config(name, args, dev, headline):
         "padded_tflops": f_pad / t_med / 1e12,
         "hbm_min_gbps": b_min / t_med / 1e9, "hbm_min_frac": b_min / t_med / 1e9 / PEAK_HBM_GBPS,
         "gather_gbps": b_gather / t_med / 1e9,
+        "gather_l1_frac": b_gather / t_med / 1e9 / PEAK_L1_GBPS,
         "preprocess_ms": pre_ms, "preprocess_gedges_per_s": E / pre_ms / 1e6,
         "preprocess_hbm_frac": pre_hbm_frac,
         "schedule": schedule,

@@ -112,6 +112,27 @@ def test_long_windows_one_bitset_pass(oracle_mod, W, seed, N, deg, messy, empty)
 
 
 @pytest.mark.parametrize("W", [16, 8])
+def test_long_windows_on_a_tiny_node_set(oracle_mod, W):
+    """Three windows of 48 nodes whose rows repeat every column dozens of times (2 400 entries per
+    row, shuffled): long windows by edge count, a bitset of one 128-bit group, every window on
+    the general path; then the same with N = 16 and sorted rows of repeats."""
+    print("case long windows, tiny N, W=%d" % W, flush=True)
+    rng = np.random.default_rng(3)
+    N = 48
+    rows = [rng.permutation(np.tile(np.arange(N, dtype=np.int32), 50)) for _ in range(N)]
+    rowPtr = np.arange(N + 1, dtype=np.int32) * (50 * N)
+    colIdx = np.concatenate(rows)
+    got = run_gpu(rowPtr, colIdx, N, W)
+    compare_preprocess(got, oracle_mod.preprocess(rowPtr, colIdx, N, 16, W))
+    N = 16
+    rows = [np.sort(rng.integers(0, N, size=300)).astype(np.int32) for _ in range(N)]
+    rowPtr = np.arange(N + 1, dtype=np.int32) * 300
+    colIdx = np.concatenate(rows)
+    got = run_gpu(rowPtr, colIdx, N, W)
+    compare_preprocess(got, oracle_mod.preprocess(rowPtr, colIdx, N, 16, W))
+
+
+@pytest.mark.parametrize("W", [16, 8])
 def test_long_windows_with_a_window_of_several_lds_chunks(oracle_mod, W):
     """As above with one window of ~55 000 distinct columns (more TC blocks than the bitmaps'
     share of LDS holds at once) and, with `messy`, the same window on the general path."""
