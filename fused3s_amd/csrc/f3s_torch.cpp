@@ -108,7 +108,7 @@ preprocess_gpu(torch::Tensor edgeList, torch::Tensor nodePointer, int num_nodes,
                             reinterpret_cast<uint64_t*>(tcbBitMap.data_ptr()), current_stream()),
         "f3s_preprocess_fill");
   } else {
-    // one call: the block arrays are allocated for the bound on the block total and returned as
+    // one call: the nTCB-sized arrays are allocated for the bound on the block total and returned as
     // views of their first nTcb entries, so the host waits for the device once, at the end
     TORCH_CHECK(blockSize_h == 16 && (blockSize_w == 16 || blockSize_w == 8),
                 "preprocess_gpu: block ", blockSize_h, "x", blockSize_w,

@@ -114,7 +114,7 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
  * a caller of this entry allocates them for f3s_preprocess_capacity(N, E, W) blocks beforehand
  * and uses the first nTCB entries.
  *
- *   capacity       TC blocks the five block arrays below have room for; at least
+ *   capacity       TC blocks the four nTCB-sized arrays below have room for; at least
  *                  f3s_preprocess_capacity(N, E, W) = ceil(E / W) + ceil(N / 16), which bounds
  *                  the total of any graph with these sizes
  *   tcblockRowid [capacity], tcblocktileId [E], tcblockOffset [capacity+1],
