@@ -50,7 +50,17 @@ __device__ __forceinline__ unsigned cu_key() {
 // blocks per step; rowWindowOffset then counts 16x8 blocks, a window may end in the middle of a
 // step, and sddmm (if not null) receives the masked, unscaled scores, row-major 16x8 per block
 // (saveSddmmResult, src/F3S_kernel.cu:99-115).
-template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS, bool W8>
+// PERSIST = true (single head, 16x16 blocks, not timed): the grid is as many workgroups as fit the
+// GPU at once; a workgroup starts at position blockIdx.x of the window order and draws every
+// further position from a device-wide cursor (the draw for the next window is in flight while the
+// current one is computed), so the order is served first come, first served without relying on
+// the order in which the hardware starts workgroups. The last workgroup to leave puts the cursor
+// back to zero: launches of this form must not overlap on one device.
+__device__ int g_windowCursor = 0;
+__device__ int g_workgroupsDone = 0;
+
+template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS, bool W8,
+          bool PERSIST = false>
 __global__ __launch_bounds__(NWAVES * 64)
 __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void f3s_fwd_kernel(
     const int32_t* __restrict__ rowWindowOffset, const int32_t* __restrict__ windowOrder,
@@ -58,7 +68,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     int nRW, int64_t nTcb, const ET* __restrict__ Q, const ET* __restrict__ K,
     const ET* __restrict__ V, float scaleLog2, float* __restrict__ out,
     unsigned long long* __restrict__ cuTimer, int nHeads, int ldIn, int ldOut,
-    float* __restrict__ sddmm, int minBlocks) {
+    float* __restrict__ sddmm, int minBlocks, int nPositions) {
   typedef pipe::PairPipeline<ET, D, SOFTMAX, HEADS, W8> Pipe;
   constexpr int T = D / 16;
   constexpr int OSTRIDE = D + 4;
@@ -67,15 +77,24 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   unsigned long long tBegin = 0;
   if constexpr (CLOCKED) tBegin = realtime_ticks();
 
-  const int pos = HEADS ? (int)(blockIdx.x / (unsigned)nHeads) : (int)blockIdx.x;
+  static_assert(!PERSIST || (!CLOCKED && !HEADS && !W8), "the persistent form is single-head");
+  __shared__ int sNextPos[2];
+  int pos = HEADS ? (int)(blockIdx.x / (unsigned)nHeads) : (int)blockIdx.x;
   const int head = HEADS ? (int)(blockIdx.x - (unsigned)pos * (unsigned)nHeads) : 0;
-  const int w = windowOrder ? windowOrder[pos] : pos;
-  if ((unsigned)w >= (unsigned)nRW) return;  // a corrupt order entry must not index out of range
   const int pitchOut = HEADS ? ldOut : D;
   const int lane = threadIdx.x & 63;
   const int wave = pipe::uniform(threadIdx.x >> 6);
   const int g = lane >> 4;
   const int c = lane & 15;
+  for (int iter = 0;; iter++) {
+  if constexpr (PERSIST) {
+    if (pos >= nPositions) break;
+    // position of the window after this one; read at the end of this iteration
+    if (threadIdx.x == 0) sNextPos[iter & 1] = atomicAdd(&g_windowCursor, 1) + (int)gridDim.x;
+  }
+  do {
+  const int w = windowOrder ? windowOrder[pos] : pos;
+  if ((unsigned)w >= (unsigned)nRW) break;  // a corrupt order entry must not index out of range
 
   int t0 = rowWindowOffset[w];
   int t1 = rowWindowOffset[w + 1];
@@ -84,7 +103,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   if (t0 < 0 || (int64_t)t1 > nTcb || t1 < t0) t1 = t0;
   // windows of at most minBlocks blocks belong to the wave-per-window kernel of the same call
   // (f3s_fwd_unit_kernel); -1 when this kernel computes every window
-  if (t1 - t0 <= minBlocks) return;
+  if (t1 - t0 <= minBlocks) break;
   const int nSteps = (t1 - t0 + BPS - 1) / BPS;
 
   pipe::Problem<ET> pb;
@@ -167,6 +186,17 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     }
     *reinterpret_cast<float4*>(out + row * pitchOut + head * D + cv * 4) = acc;
   }
+  } while (false);
+  if constexpr (!PERSIST) break;
+  __syncthreads();  // the merge buffers are free again, the next position has arrived
+  pos = sNextPos[iter & 1];
+  }
+  if constexpr (PERSIST) {
+    if (threadIdx.x == 0 && atomicAdd(&g_workgroupsDone, 1) == (int)gridDim.x - 1) {
+      atomicExch(&g_windowCursor, 0);
+      atomicExch(&g_workgroupsDone, 0);
+    }
+  }
   if constexpr (CLOCKED) {
     // {first tick, last tick, CU} of this workgroup, as the reference's timed kernels record
     // {begin, end, smid} per block (src/F3S_kernel.cu:1363-1367)
@@ -186,6 +216,13 @@ int allow_lds(KernelT kernel, size_t bytes) {
     F3S_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
   return 0;
+}
+
+// F3S_WINDOW_PERSISTENT=1 in the environment (read per call): the workgroup-per-window kernel in
+// its cursor form
+bool window_cursor_requested() {
+  const char* e = getenv("F3S_WINDOW_PERSISTENT");
+  return e && strcmp(e, "1") == 0;
 }
 
 struct HeadLayout {
@@ -219,14 +256,30 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
     hipLaunchKernelGGL(kernel, dim3(GRID), block, lds, stream, rwo, order, atox, bm, N, nRW,    \
                        hl.nTcb, q, k, v, scaleLog2, out, cuTimer, hl.nHeads > 0 ? hl.nHeads : 1,\
                        hl.nHeads > 0 ? hl.ldIn : D, hl.nHeads > 0 ? hl.ldOut : D,               \
-                       (float*)nullptr, hl.minBlocks);                                          \
+                       (float*)nullptr, hl.minBlocks, (int)gw);                                 \
   }
-  if (hl.nHeads > 0)
+  if (hl.nHeads > 0) {
     F3S_LAUNCH(false, true, gw * (unsigned)hl.nHeads)
-  else if (cuTimer)
+  } else if (cuTimer) {
     F3S_LAUNCH(true, false, gw)
-  else
+  } else if (window_cursor_requested()) {
+    // F3S_WINDOW_PERSISTENT=1: as many workgroups as the GPU holds at once, windows drawn from a
+    // cursor (measured slower than launch order, which therefore stays the default)
+    auto kernel = f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false, false, true>;
+    if (int rc = allow_lds(kernel, lds)) return rc;
+    int dev = 0, nCu = 0, perCu = 0;
+    F3S_HIP_CHECK(hipGetDevice(&dev));
+    F3S_HIP_CHECK(hipDeviceGetAttribute(&nCu, hipDeviceAttributeMultiprocessorCount, dev));
+    F3S_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+        &perCu, reinterpret_cast<const void*>(kernel), NWAVES * 64, lds));
+    unsigned grid = (unsigned)(nCu * (perCu > 0 ? perCu : 1));
+    if (grid > gw) grid = gw;
+    hipLaunchKernelGGL(kernel, dim3(grid), block, lds, stream, rwo, order, atox, bm, N, nRW,
+                       hl.nTcb, q, k, v, scaleLog2, out, cuTimer, 1, D, D, (float*)nullptr,
+                       hl.minBlocks, (int)gw);
+  } else {
     F3S_LAUNCH(false, false, gw)
+  }
 #undef F3S_LAUNCH
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
@@ -245,7 +298,8 @@ int launch_tcb8(const int32_t* rwo, const int32_t* order, const int32_t* atox,
   hipLaunchKernelGGL(kernel, dim3(nRW), dim3(NWAVES * 64), lds, stream, rwo, order, atox,
                      reinterpret_cast<const uint8_t*>(bitmap), N, nRW, nTcb8,
                      static_cast<const _Float16*>(Q), static_cast<const _Float16*>(K),
-                     static_cast<const _Float16*>(V), scaleLog2, out, nullptr, 1, D, D, sddmm, -1);
+                     static_cast<const _Float16*>(V), scaleLog2, out, nullptr, 1, D, D, sddmm, -1,
+                     nRW);
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
@@ -298,9 +352,9 @@ bool split_short_windows(const int32_t* windowOrder, int nRW, int64_t nTcb, Head
 
 // The column-sliced schedule (f3s_attention_units.hip: (window, column slice) units, every XCD
 // on one slice at a time so that its K/V rows stay in that XCD's L2, plus a merge kernel) pays off
-// on graphs with long windows: on the 233k-node benchmark graph (475 TC blocks per window) it
-// takes 1.66 / 1.94 / 3.67 ms at d = 32 / 64 / 128 against 2.27 / 2.11 / 6.05 ms for the
-// workgroup-per-window kernel, with 6.5 GB instead of 15.1 GB of traffic beyond L2 at d = 64.
+// on graphs with long windows: on the 233k-node benchmark graph (450 TC blocks per window) it
+// takes 1.54 ms at d = 64 against 2.48 ms for the workgroup-per-window kernel, with 7.1 GB
+// instead of 17.7 GB of traffic beyond L2.
 // Short windows would be cut into units of one or two blocks; they keep the window kernel.
 // F3S_SCHEDULE=window / =sliced in the environment overrides the choice.
 int attention_uses_workspace(int N, int64_t nTcb, int d, int dtype) {

@@ -160,6 +160,29 @@ def test_column_sliced_schedule_with_several_phases(oracle_mod, monkeypatch, pha
         assert mean_rel(got, want) < MEAN_REL
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_window_kernel_with_a_cursor_gives_the_same_rows(monkeypatch, d):
+    """The workgroup-per-window kernel as a resident grid that draws windows from a device-wide
+    cursor (F3S_WINDOW_PERSISTENT=1) against its launch-ordered form: the same arithmetic per
+    window, so bit-identical rows; three calls in a row (the cursor is put back by the kernel),
+    with and without an order, on more windows than workgroups fit the GPU (4 000)."""
+    print("case window cursor d=%d" % d, flush=True)
+    import oracle
+    oracle.build()
+    rng = np.random.default_rng(d)
+    N = 64_000
+    rowPtr, colIdx = random_csr(rng, N, 6, hub=997, empty_frac=0.02)
+    Q, K, V = feats(rng, N, d)
+    pre = oracle.preprocess(rowPtr, colIdx, N)
+    order = pre["sortedRowWindows"]
+    for od in (order, None, order):
+        monkeypatch.setenv("F3S_WINDOW_PERSISTENT", "0")
+        want = gpu_attention(pre, N, Q, K, V, 8.0, od)
+        monkeypatch.setenv("F3S_WINDOW_PERSISTENT", "1")
+        got = gpu_attention(pre, N, Q, K, V, 8.0, od)
+        assert np.isfinite(want).all() and np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("d", [32, 64])
 def test_column_sliced_schedule_matches_oracle_and_window_kernel(oracle_mod, d):
     """The column-sliced schedule on a dense power-law graph (>= 2048 windows, >= 64 TC blocks per
