@@ -35,6 +35,9 @@ using pipe::uniform;
 constexpr int kXcds = 8;
 constexpr int kMaxPhases = 16;
 constexpr int kUnitWaves = 4;  // waves (= units) per workgroup; they do not cooperate
+// the same for the wave-per-window launches of graphs with short windows (measured on the 100k-node
+// 8-head layers: 0.093 / 0.171 ms with two, 0.099 / 0.175 ms with four, 0.121 / 0.197 ms with one)
+constexpr int kShortUnitWaves = 2;
 constexpr int kQueueBatch = 8;  // units a persistent wave takes per visit to a queue
 
 // sliceStart[w * (S + 1) + s] = first TC block of window w whose first (smallest) column id is
@@ -113,7 +116,7 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
     const int xcd = blockIdx.x % kXcds;
     const int j = blockIdx.x / kXcds;
     const int phase = j / nGroups;
-    const int pos = (j - phase * nGroups) * kUnitWaves + wave;
+    const int pos = (j - phase * nGroups) * (int)(blockDim.x >> 6) + wave;
     if (pos >= nRW) return;
     slice = phase * kXcds + xcd;
     w = uniform(windowOrder ? windowOrder[pos] : pos);
@@ -122,7 +125,7 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
     t1 = uniform(sliceStart[(int64_t)w * (S + 1) + slice + 1]);
     if (t1 <= t0) return;  // empty unit: nothing is written, the merge skips it
   } else {
-    const int64_t u = (int64_t)blockIdx.x * kUnitWaves + wave;
+    const int64_t u = (int64_t)blockIdx.x * (int)(blockDim.x >> 6) + wave;
     const int pos = HEADS ? (int)(u / nHeads) : (int)u;
     head = HEADS ? (int)(u - (int64_t)pos * nHeads) : 0;
     if (pos >= nRW) return;
@@ -505,12 +508,13 @@ int launch_short_d(const int32_t* rwo, const int32_t* order, const int32_t* atox
                    int longPrefix, int64_t nTcb, hipStream_t stream) {
   const int64_t nRW = ((int64_t)N + kWinRows - 1) / kWinRows;
   const int64_t units = nRW * (nHeads > 0 ? nHeads : 1);
-  const dim3 grid((unsigned)((units + kUnitWaves - 1) / kUnitWaves)), block(kUnitWaves * 64);
+  const dim3 grid((unsigned)((units + kShortUnitWaves - 1) / kShortUnitWaves)),
+      block(kShortUnitWaves * 64);
   const auto* bm = reinterpret_cast<const uint8_t*>(bitmap);
   const auto* q = static_cast<const ET*>(Q);
   const auto* k = static_cast<const ET*>(K);
   const auto* v = static_cast<const ET*>(V);
-  constexpr size_t lds = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES;
+  constexpr size_t lds = (size_t)kShortUnitWaves * pipe::Geo<D>::WAVE_BYTES;
   if (nHeads > 0) {
     if (int rc = allow_lds(f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, true>, lds)) return rc;
     hipLaunchKernelGGL((f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, true>), grid, block, lds,
