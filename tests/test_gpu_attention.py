@@ -160,6 +160,36 @@ def test_column_sliced_schedule_with_several_phases(oracle_mod, monkeypatch, pha
         assert mean_rel(got, want) < MEAN_REL
 
 
+def test_windows_beyond_the_stated_block_total_are_left_empty(oracle_mod):
+    """A caller that states fewer TC blocks than rowWindowOffset ends with (for instance the arrays
+    of another preprocessing run): windows whose block range ends beyond the stated total are
+    treated as empty (rows of zeros) instead of being followed; the others are computed as usual.
+    The arrays passed here are views of the full ones, so every address stays valid either way."""
+    print("case stated block total", flush=True)
+    from fused3s_amd import capi
+    rng = np.random.default_rng(21)
+    N, d = 4000, 64
+    rowPtr, colIdx = random_csr(rng, N, 30)
+    Q, K, V = feats(rng, N, d)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    full = gpu_attention(pre, N, Q, K, V, 8.0)
+    rwo = pre["rowWindowOffset"]
+    keep = int(np.searchsorted(rwo, rwo[-1] // 2, side="right")) - 1  # windows wholly in the first half
+    stated = int(rwo[keep])
+    dev = "cuda"
+    atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)[: stated * 16]
+    bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)[: stated * 4]
+    for order in (None, pre["sortedRowWindows"]):
+        od = None if order is None else torch.as_tensor(np.asarray(order, np.int32)).to(dev)
+        out = capi.attention(torch.as_tensor(rwo.astype(np.int32)).to(dev), od, atox, bm, N,
+                             torch.as_tensor(Q).to(dev), torch.as_tensor(K).to(dev),
+                             torch.as_tensor(V).to(dev), 8.0)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.array_equal(got[: keep * 16], full[: keep * 16])
+        assert not got[keep * 16:].any()
+
+
 @pytest.mark.parametrize("d", [32, 64, 128])
 def test_window_kernel_with_a_cursor_gives_the_same_rows(monkeypatch, d):
     """The workgroup-per-window kernel as a resident grid that draws windows from a device-wide
