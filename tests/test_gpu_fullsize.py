@@ -40,6 +40,25 @@ def check_close(got, want, what):
     assert rel < MEAN_REL, (what, rel)
 
 
+def test_preprocessing_at_the_largest_single_pass_column_range(oracle_mod):
+    """N = 393 216 nodes (the most columns one LDS bitset holds) and 53 M edges: the kernel that
+    does both phases per window runs with its largest bitset, which leaves room for 224 TC blocks
+    of bitmaps at a time, so every window takes several chunks. One node more and the same call
+    takes the multi-pass kernels. Both must match the oracle bit for bit (and count / fill)."""
+    from fused3s_amd import capi, synth
+    for N in (393_216, 393_217):
+        print("case single-pass limit N=%d" % N, flush=True)
+        rowPtr, colIdx = synth.chung_lu_graph(N, 53_000_000, gamma=2.3, max_degree=6000, seed=3,
+                                              device="cuda")
+        E = colIdx.numel()
+        assert E >= ((N + 15) // 16) * 2048
+        want = oracle_mod.preprocess(rowPtr.cpu().numpy(), colIdx.cpu().numpy(), N)
+        for two_phase in (False, True):
+            got = host(capi.preprocess(rowPtr, colIdx, N, two_phase=two_phase))
+            compare_preprocess(got, want)
+        del want, got
+
+
 @pytest.mark.parametrize("name", ["cfg3_chunglu_233k", "cfg4_rmat_2449k"])
 def test_full_size_graph(oracle_mod, name):
     from fused3s_amd import capi, synth
