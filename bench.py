@@ -159,12 +159,13 @@ def run_config(name, args, dev, headline):
     scale = float(np.sqrt(d))
 
     # preprocessing (timed on its own; not part of the step)
-    capi.preprocess(rowPtr, colIdx, N)  # warm-up (module load, allocator)
+    two_phase = bool(getattr(args, "two_phase_preprocess", False))
+    capi.preprocess(rowPtr, colIdx, N, two_phase=two_phase)  # warm-up (module load, allocator)
     torch.cuda.synchronize()
     pre_ms = []
     for _ in range(3):
         t0 = time.time()
-        pre = capi.preprocess(rowPtr, colIdx, N)
+        pre = capi.preprocess(rowPtr, colIdx, N, two_phase=two_phase)
         torch.cuda.synchronize()
         pre_ms.append((time.time() - t0) * 1e3)
     pre_ms = float(np.median(pre_ms))
@@ -335,6 +336,9 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the compact lines of the other benchmark configurations")
     ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
+    ap.add_argument("--two-phase-preprocess", action="store_true",
+                    help="preprocess with f3s_preprocess_count + f3s_preprocess_fill instead of "
+                         "the one call f3s_preprocess")
     ap.add_argument("--cpu-budget", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
