@@ -162,6 +162,37 @@ def test_long_windows_quarter_scale_benchmark_graph(oracle_mod):
     compare_preprocess(got, want)
 
 
+def test_sweep_of_random_shapes(oracle_mod):
+    """Forty seeded graphs of mixed shapes (node counts around multiples of 16 and 128, short and
+    long windows, repeated / shuffled / empty rows, hub rows, both block widths) through both
+    entry styles against the oracle."""
+    rng = np.random.default_rng(2024)
+    for it in range(40):
+        W = 16 if it % 3 else 8
+        N = int(rng.choice([15, 16, 17, 127, 128, 129, 500, 1023, 2049, 4100]))
+        long_windows = it % 4 == 0
+        if long_windows:
+            deg = int(rng.integers(140, 400))
+            messy = int(rng.choice([0, 1, 7, 50]))
+            rowPtr, colIdx = long_window_graph(rng, N, deg, messy_every=messy,
+                                               empty_every=int(rng.choice([0, 9])))
+            if messy == 1 or rowPtr[-1] < ((N + 15) // 16) * 2048:
+                # repeats push short rows of a small node set over the long-window threshold
+                rep = int(np.ceil(((N + 15) // 16) * 2048 / max(1, rowPtr[-1]))) + 1
+                rows = [np.tile(colIdx[rowPtr[r]:rowPtr[r + 1]], rep) for r in range(N)]
+                rowPtr = np.zeros(N + 1, np.int32)
+                rowPtr[1:] = np.cumsum([len(x) for x in rows])
+                colIdx = np.concatenate(rows).astype(np.int32)
+        else:
+            rowPtr, colIdx = random_csr(rng, N, int(rng.integers(1, 40)), dup=bool(it & 1),
+                                        unsorted=bool(it & 2), empty_frac=float(rng.choice([0, 0.3])),
+                                        hub=int(rng.choice([0, 11])))
+        print("case sweep %d: N=%d E=%d W=%d long=%s" % (it, N, rowPtr[-1], W, long_windows),
+              flush=True)
+        got = run_gpu(rowPtr, colIdx, N, W)
+        compare_preprocess(got, oracle_mod.preprocess(rowPtr, colIdx, N, 16, W))
+
+
 def test_heavy_window_many_blocks(oracle_mod):
     """One window whose rows name > 16*512 distinct columns: several LDS chunks in the fill."""
     print("case heavy_window", flush=True)
