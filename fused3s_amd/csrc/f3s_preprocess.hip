@@ -92,6 +92,47 @@ __device__ __forceinline__ int row_of_edge(const int* sRow, int e) {
   return r;
 }
 
+// Writes a TC block's tile ids (row * W + column of every set bit, rows top to bottom, columns
+// left to right) to dst[pos...]. words: the block's bitmap, 8x8 sub-blocks in column-major order,
+// rows of a sub-block MSB first. The bitmap is first brought into row-major order as dwords whose
+// bit 31 - p stands for tile id 32 q + p (two rows of 16 columns, or four of 8, per dword): for
+// 16 columns that interleaves the bytes of the left and the right sub-block (two byte permutes
+// per four rows), for 8 columns the words are in that order already.
+template <int W>
+__device__ __forceinline__ void walk_tile_ids(const unsigned long long (&words)[16 * W / 64],
+                                              uint8_t* __restrict__ dst, unsigned pos) {
+  constexpr int NQ = 16 * W / 32;
+  unsigned rm[NQ];
+  if constexpr (W == 16) {
+#pragma unroll
+    for (int half = 0; half < 2; half++) {  // rows 0-7 (sub-blocks 0 and 2), rows 8-15 (1 and 3)
+      const unsigned long long left = words[half], right = words[2 + half];
+#pragma unroll
+      for (int k = 0; k < 2; k++) {  // rows 4k .. 4k+3 of the half: the dword from the top
+        const unsigned a = k == 0 ? (unsigned)(left >> 32) : (unsigned)left;
+        const unsigned c = k == 0 ? (unsigned)(right >> 32) : (unsigned)right;
+        rm[4 * half + 2 * k] = __builtin_amdgcn_perm(a, c, 0x07030602u);      // rows +0, +1
+        rm[4 * half + 2 * k + 1] = __builtin_amdgcn_perm(a, c, 0x05010400u);  // rows +2, +3
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      rm[2 * k] = (unsigned)(words[k] >> 32);
+      rm[2 * k + 1] = (unsigned)words[k];
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < NQ; q++) {
+    unsigned x = rm[q];
+    while (x) {
+      const int p = __builtin_clz(x);
+      dst[pos++] = (uint8_t)(32 * q + p);
+      x &= ~(0x80000000u >> p);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ phase 1
 // compiler-level ordering point between LDS phases of ONE wave (its LDS operations execute in
 // program order, so no hardware barrier is needed)
@@ -1003,20 +1044,7 @@ __device__ __forceinline__ void fill_window_generic(
           unsigned long long words[WPT];
 #pragma unroll
           for (int k = 0; k < WPT; k++) words[k] = sBm[t * WPT + k];
-          unsigned pos = run;
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            unsigned rowBits = 0;  // W bits, column 0 in the most significant one
-#pragma unroll
-            for (int h = 0; h < W / 8; h++)
-              rowBits = (rowBits << 8) |
-                        ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
-            while (rowBits) {
-              const int cl = __clz(rowBits) - (32 - W);
-              tcblocktileId[pos++] = (uint8_t)(r * W + cl);
-              rowBits &= ~(1u << (W - 1 - cl));
-            }
-          }
+          walk_tile_ids<W>(words, tcblocktileId, run);
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -1235,19 +1263,7 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
         tcblockRowid[gt] = w;
         // tile ids: the block's set bits read row by row (each lane walks its own block; the
         // byte stores of neighbouring lanes fall next to each other)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          unsigned rowBits = 0;  // W bits, column 0 in the most significant one
-#pragma unroll
-          for (int h = 0; h < W / 8; h++)
-            rowBits = (rowBits << 8) |
-                      ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
-          while (rowBits) {
-            const int cl = __clz(rowBits) - (32 - W);
-            tcblocktileId[pos++] = (uint8_t)(r * W + cl);
-            rowBits &= ~(1u << (W - 1 - cl));
-          }
-        }
+        walk_tile_ids<W>(words, tcblocktileId, pos);
       }
       carry += tileTot;
       __syncthreads();
@@ -1292,26 +1308,6 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
 // talk to each other through LDS and never through global memory.
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// Writes a TC block's tile ids (row * W + column of every set bit, rows top to bottom, columns
-// left to right) to dst[pos...]. words: the block's bitmap, 8x8 sub-blocks in column-major order.
-template <int W>
-__device__ __forceinline__ void walk_tile_ids(const unsigned long long (&words)[16 * W / 64],
-                                              uint8_t* __restrict__ dst, unsigned pos) {
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    unsigned rowBits = 0;  // W bits, column 0 in the most significant one
-#pragma unroll
-    for (int h = 0; h < W / 8; h++)
-      rowBits = (rowBits << 8) |
-                ((unsigned)(words[h * (W / 8) + (r >> 3)] >> (8 * (7 - (r & 7)))) & 0xFFu);
-    while (rowBits) {
-      const int cl = __clz(rowBits) - (32 - W);
-      dst[pos++] = (uint8_t)(r * W + cl);
-      rowBits &= ~(1u << (W - 1 - cl));
-    }
-  }
 }
 
 // The window's edges [eS, eE) as whole 4-aligned groups [gA, gB) plus the edges in front of and
