@@ -163,7 +163,7 @@ def run_config(name, args, dev, headline):
     capi.preprocess(rowPtr, colIdx, N, two_phase=two_phase)  # warm-up (module load, allocator)
     torch.cuda.synchronize()
     pre_ms = []
-    for _ in range(3):
+    for _ in range(7):
         t0 = time.time()
         pre = capi.preprocess(rowPtr, colIdx, N, two_phase=two_phase)
         torch.cuda.synchronize()
