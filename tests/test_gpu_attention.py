@@ -160,6 +160,57 @@ def test_column_sliced_schedule_with_several_phases(oracle_mod, monkeypatch, pha
         assert mean_rel(got, want) < MEAN_REL
 
 
+def test_sweep_of_random_problems(oracle_mod):
+    """Thirty seeded problems of mixed shape (node counts around multiples of 16, degrees from 1 to
+    a few hundred, hub rows, empty rows), head dimension, input type (fp16 / bf16), window order and
+    score scaling (fp16 also unscaled, where rows of very negative scores underflow to 0 as in the
+    reference) through f3s_attention_fwd against the reference-emulating oracle, every tenth one
+    without softmax."""
+    from fused3s_amd import capi
+    rng = np.random.default_rng(77)
+    dev = "cuda"
+    as_bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
+    for it in range(30):
+        N = int(rng.choice([16, 17, 31, 100, 257, 1000, 3001]))
+        d = int(rng.choice([32, 64, 128]))
+        deg = int(rng.choice([1, 3, 17, 60, 250]))
+        deg = min(deg, max(1, N // 2))
+        bf16 = bool(it % 3 == 1)
+        softmax = it % 10 != 9
+        scale = float(rng.choice([1.0, np.sqrt(d)]))
+        if bf16:
+            # unscaled scores of N(0, d) reach below -17, where the reference's fp16 probabilities
+            # underflow to 0 (a row of only such scores comes out as 0, which the fp16 kernel
+            # reproduces); the bf16 kernel keeps them, so it is compared where they survive
+            scale = float(np.sqrt(d))
+        rowPtr, colIdx = random_csr(rng, N, deg, hub=int(rng.choice([0, 13])),
+                                    empty_frac=float(rng.choice([0.0, 0.2])))
+        print("case sweep %d: N=%d d=%d deg=%d bf16=%s softmax=%s scale=%.2f"
+              % (it, N, d, deg, bf16, softmax, scale), flush=True)
+        std = 1.0 if softmax else 0.4
+        Qf, Kf, Vf = [(rng.standard_normal((N, d)) * std).astype(np.float32) for _ in range(3)]
+        tdt = torch.bfloat16 if bf16 else torch.float16
+        Qt, Kt, Vt = (torch.as_tensor(x).to(tdt) for x in (Qf, Kf, Vf))
+        pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+        if bf16:
+            want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                            pre["tcbBitMap"], N, as_bits(Qt), as_bits(Kt),
+                                            as_bits(Vt), scale, applySoftmax=softmax, dtype=1)
+        else:
+            want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                            pre["tcbBitMap"], N, Qt.numpy(), Kt.numpy(),
+                                            Vt.numpy(), scale, applySoftmax=softmax)
+        rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
+        atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
+        bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
+        od = torch.as_tensor(pre["sortedRowWindows"].astype(np.int32)).to(dev) if it & 1 else None
+        got = capi.attention(rwo, od, atox, bm, N, Qt.to(dev), Kt.to(dev), Vt.to(dev), scale,
+                             softmax).cpu().numpy()
+        assert np.isfinite(got).all()
+        assert np.abs(got - want).max() < MAX_ABS * (1.0 if softmax else max(1.0, np.abs(want).max()))
+        assert mean_rel(got, want) < MEAN_REL
+
+
 def test_windows_beyond_the_stated_block_total_are_left_empty(oracle_mod):
     """A caller that states fewer TC blocks than rowWindowOffset ends with (for instance the arrays
     of another preprocessing run): windows whose block range ends beyond the stated total are
