@@ -108,6 +108,41 @@ def test_reference_call_sequence_all_variants(oracle_mod, tmp_path, monkeypatch)
             assert float(e) >= float(b) > 0
 
 
+@pytest.mark.parametrize("W", [16, 8])
+def test_preprocess_gpu_both_allocation_styles(oracle_mod, monkeypatch, W):
+    """F3S.preprocess_gpu with views of bounded allocations (default) and with the reference's
+    count / allocate / fill sequence (F3S_PREPROCESS=two_phase): the same tuples, bit for bit, on a
+    graph of long windows and on one of short windows; the default's tensors are contiguous views
+    whose sizes are the exact ones."""
+    from fused3s_amd import F3S
+    from test_gpu_preprocess import long_window_graph
+    rng = np.random.default_rng(5)
+    graphs = [long_window_graph(rng, 2000, 180, messy_every=60, empty_every=13)]
+    rp, ci, _, _, _ = reference_style_inputs(1000, 32)
+    graphs.append((rp, ci))
+    for rowPtr, colIdx in graphs:
+        N = len(rowPtr) - 1
+        print("case module allocation styles N=%d E=%d W=%d" % (N, len(colIdx), W), flush=True)
+        want = oracle_mod.preprocess(rowPtr, colIdx, N, 16, W)
+        results = []
+        for style in ("", "two_phase"):
+            monkeypatch.setenv("F3S_PREPROCESS", style)
+            res, bp, e2c, e2r = preprocess_like_the_reference(F3S, rowPtr, colIdx, N, W)
+            rwo, order, rowid, tile, toff, atox, bm, count = res
+            assert count == want["blockCount"]
+            assert rowid.numel() == count and toff.numel() == count + 1
+            assert atox.numel() == count * W and bm.numel() == count * 16 * W // 64
+            assert all(t.is_contiguous() for t in (rowid, toff, atox, bm, tile))
+            got = dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
+                       tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox,
+                       blockCount=count,
+                       tcbBitMap=bm.cpu().view(torch.int64).numpy().view(np.uint64),
+                       blockPartition=bp, edgeToColumn=e2c, edgeToRow=e2r)
+            got = {k: (v.cpu().numpy() if torch.is_tensor(v) else v) for k, v in got.items()}
+            compare_preprocess(got, want)
+            results.append(got)
+
+
 def test_module_argument_checks_on_device():
     print("case module_arg_checks", flush=True)
     from fused3s_amd import F3S
