@@ -191,7 +191,12 @@ def run_config(name, args, dev, headline):
     order = None if natural else pre["sortedRowWindows"]
     out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
     # scratch of the column-sliced schedule, which the library picks for graphs with long windows
-    workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype) if heads == 1 else None
+    workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype,
+                                         heads=0 if heads == 1 else heads)
+    if workspace is not None:
+        # the schedule's index depends on the structure only: built once, like the structure
+        capi.attention_prepare(pre["rowWindowOffset"], pre["sparseAToXidx"], N, d,
+                               workspace, heads=0 if heads == 1 else heads)
     schedule = "column-sliced" if workspace is not None else "window"
     log("attention schedule: %s" % ("column-sliced (%.0f MB workspace)" % (workspace.numel() / 1e6)
                                     if workspace is not None else "workgroup per window"))
@@ -199,11 +204,13 @@ def run_config(name, args, dev, headline):
     if heads == 1:
         def step(v=V, o=out):
             capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"], pre["tcbBitMap"],
-                           N, Q, K, v, scale, True, out=o, workspace=workspace)
+                           N, Q, K, v, scale, True, out=o, workspace=workspace,
+                           prepared=workspace is not None)
     else:
         def step(v=V, o=out):
             capi.attention_heads(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
-                                 pre["tcbBitMap"], N, Q, K, v, scale, True, out=o)
+                                 pre["tcbBitMap"], N, Q, K, v, scale, True, out=o,
+                                 workspace=workspace, prepared=workspace is not None)
 
     steps, warmup = (args.steps, args.warmup) if headline else (10, 3)
     for _ in range(warmup):

@@ -17,9 +17,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libf3s_amd.so")
 EXT_PATH = os.path.join(HERE, "F3S" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
-HIP_SOURCES = ["f3s_capi.hip", "f3s_attention.hip", "f3s_attention_units.hip", "f3s_preprocess.hip"]
+HIP_SOURCES = ["f3s_capi.hip", "f3s_attention.hip", "f3s_attention_wide.hip",
+               "f3s_attention_units.hip", "f3s_preprocess.hip"]
 HIP_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
     # packed-fp32 code generation is switched off for every device translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
@@ -45,31 +46,49 @@ PROBES = {
 }
 
 
-def build_probe(name):
+def _compile_and_link(out, extra_flags, tag):
+    """Every translation unit in its own hipcc process (they are independent and take most of the
+    time), then one link. Objects go to build/<tag>/ and are rebuilt every time."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    out_dir = os.path.join(HERE, "probes")
-    os.makedirs(out_dir, exist_ok=True)
-    out = os.path.join(out_dir, "libf3s_amd_%s.so" % name)
-    _run([hipcc] + HIP_FLAGS + PROBES[name] + ["-o", out] + srcs)
+    obj_dir = os.path.join(HERE, "build", tag)
+    os.makedirs(obj_dir, exist_ok=True)
+    jobs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc] + HIP_FLAGS + extra_flags + ["-c", os.path.join(CSRC, src), "-o", obj]
+        jobs.append((cmd, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE,
+                                                stderr=subprocess.STDOUT, text=True)))
+    objs = []
+    for cmd, obj, proc in jobs:
+        _report(cmd, proc.communicate()[0], proc.returncode)
+        objs.append(obj)
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
     return out
 
 
-def _run(cmd):
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines()
+def build_probe(name):
+    out_dir = os.path.join(HERE, "probes")
+    os.makedirs(out_dir, exist_ok=True)
+    out = os.path.join(out_dir, "libf3s_amd_%s.so" % name)
+    return _compile_and_link(out, PROBES[name], "probe_" + name)
+
+
+def _report(cmd, text, returncode):
+    out = "\n".join(l for l in text.splitlines()
                     if "not a recognized feature for this target" not in l)
-    if proc.returncode != 0:
+    if returncode != 0:
         raise RuntimeError("build failed: %s\n%s" % (" ".join(cmd), out))
     if out.strip():
         print(out)
 
 
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    _report(cmd, proc.stdout, proc.returncode)
+
+
 def build_library():
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    _run([hipcc] + HIP_FLAGS + ["-o", LIB_PATH] + srcs)
-    return LIB_PATH
+    return _compile_and_link(LIB_PATH, [], "lib")
 
 
 def build_extension():

@@ -18,7 +18,8 @@ EXPORTS = ["f3s_abi_version", "f3s_last_error", "f3s_preprocess_workspace_bytes"
            "f3s_attention_workspace_bytes", "f3s_attention_fwd_heads",
            "f3s_attention_fwd_tcb8", "f3s_attention_uses_workspace",
            "f3s_preprocess_static_scratch_bytes", "f3s_preprocess_count_static",
-           "f3s_preprocess_capacity", "f3s_preprocess"]
+           "f3s_preprocess_capacity", "f3s_preprocess", "f3s_attention_prepare",
+           "f3s_attention_heads_workspace_bytes", "f3s_attention_uses_wide_offsets"]
 
 
 def lib():
@@ -52,13 +53,19 @@ def lib():
                                      vp]
         L.f3s_attention_fwd.restype = ci
         L.f3s_attention_fwd.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, vp, vp, vp,
-                                        ctypes.c_float, ci, vp, vp, vp, cs, vp]
+                                        ctypes.c_float, ci, vp, vp, vp, cs, ci, vp]
         L.f3s_attention_workspace_bytes.restype = cs
         L.f3s_attention_workspace_bytes.argtypes = [ci, ci]
         L.f3s_attention_fwd_heads.restype = ci
         L.f3s_attention_fwd_heads.argtypes = [vp, vp, vp, vp, ci, ctypes.c_int64, ci, ci, ci, vp,
                                               vp, vp, ctypes.c_int64, ctypes.c_float, ci, vp,
-                                              ctypes.c_int64, vp]
+                                              ctypes.c_int64, vp, cs, ci, vp]
+        L.f3s_attention_heads_workspace_bytes.restype = cs
+        L.f3s_attention_heads_workspace_bytes.argtypes = [ci, ci, ci]
+        L.f3s_attention_prepare.restype = ci
+        L.f3s_attention_prepare.argtypes = [vp, vp, ci, ctypes.c_int64, ci, ci, vp, cs, vp]
+        L.f3s_attention_uses_wide_offsets.restype = ci
+        L.f3s_attention_uses_wide_offsets.argtypes = [ctypes.c_int64, ctypes.c_int64, ci]
         L.f3s_attention_uses_workspace.restype = ci
         L.f3s_attention_uses_workspace.argtypes = [ci, ctypes.c_int64, ci, ci]
         L.f3s_attention_fwd_tcb8.restype = ci
@@ -167,19 +174,32 @@ def preprocess_count_static(rowPtr, colIdx, N, out, H=16, W=16):
             _ptr(out["sortedRowWindows"]), _ptr(out["result"]), _stream()))
 
 
-def attention_workspace(N, d, device, nTCB=None, dtype=torch.float16):
-    """Scratch tensor for attention(..., workspace=...) (column-sliced schedule). With nTCB given,
-    returns None when the library would not use it for this problem."""
+def attention_workspace(N, d, device, nTCB=None, dtype=torch.float16, heads=0):
+    """Scratch tensor for attention(..., workspace=...) / attention_heads(..., workspace=...)
+    (column-sliced schedule; heads = 0 for the single-head call). With nTCB given, returns None
+    when the library would not use it for this problem."""
     L = lib()
     if nTCB is not None and not L.f3s_attention_uses_workspace(
             N, int(nTCB), d, 0 if dtype == torch.float16 else 1):
         return None
-    nbytes = L.f3s_attention_workspace_bytes(N, d)
-    return torch.empty(max(nbytes, 4), dtype=torch.uint8, device=device)
+    nbytes = (L.f3s_attention_heads_workspace_bytes(N, heads, d) if heads > 0
+              else L.f3s_attention_workspace_bytes(N, d))
+    return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+
+
+def attention_prepare(rwo, atox, N, d, workspace, heads=0):
+    """f3s_attention_prepare on the current stream: builds the column-sliced schedule's index in
+    `workspace` for these arrays, which must then stay unchanged while it is in use."""
+    L = lib()
+    _dev(rwo, torch.int32, "rowWindowOffset")
+    _dev(atox, torch.int32, "sparseAToXidx")
+    with torch.cuda.device(rwo.device):
+        _check(L.f3s_attention_prepare(_ptr(rwo), _ptr(atox), N, atox.numel() // 16,
+                                       d, heads, _ptr(workspace), workspace.numel(), _stream()))
 
 
 def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoftmax=True,
-              out=None, workspace=None):
+              out=None, workspace=None, prepared=False):
     """f3s_attention_fwd on the current stream; returns out fp32[N, d]."""
     L = lib()
     _dev(rwo, torch.int32, "rowWindowOffset")
@@ -210,12 +230,13 @@ def attention(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoft
                                    atox.numel() // 16, d, dtype, _ptr(Q), _ptr(K), _ptr(V),
                                    float(scalingFactor), int(bool(applySoftmax)), _ptr(out), None,
                                    _ptr(workspace),
-                                   0 if workspace is None else workspace.numel(), _stream()))
+                                   0 if workspace is None else workspace.numel(),
+                                   int(bool(prepared)), _stream()))
     return out
 
 
 def attention_heads(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, applySoftmax=True,
-                    out=None):
+                    out=None, workspace=None, prepared=False):
     """f3s_attention_fwd_heads on the current stream. Q, K, V: [N, nHeads, d] fp16 or bf16 whose
     last two dimensions are contiguous (dim 0 may be pitched); returns out fp32[N, nHeads*d]."""
     L = lib()
@@ -255,7 +276,9 @@ def attention_heads(rwo, order, atox, bitmap, N, Q, K, V, scalingFactor=1.0, app
                                          atox.numel() // 16, nHeads, d, dtype, _ptr(Q), _ptr(K),
                                          _ptr(V), Q.stride(0), float(scalingFactor),
                                          int(bool(applySoftmax)), _ptr(out), out.stride(0),
-                                         _stream()))
+                                         _ptr(workspace),
+                                         0 if workspace is None else workspace.numel(),
+                                         int(bool(prepared)), _stream()))
     return out
 
 

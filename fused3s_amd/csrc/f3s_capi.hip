@@ -26,7 +26,7 @@ bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p
 
 extern "C" {
 
-int f3s_abi_version(void) { return 1; }
+int f3s_abi_version(void) { return 2; }
 
 const char* f3s_last_error(void) { return f3s::g_error; }
 
@@ -82,8 +82,9 @@ int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int
   if (nTCB > 0 && (!tcblockRowid || !sparseAToXidx || !tcbBitMap || !colIdx || !edgeToColumn ||
                    !tcblocktileId))
     return f3s::fail(-1, "f3s_preprocess_fill: null output");
-  if (f3s::misaligned(tcbBitMap, 8))
-    return f3s::fail(-1, "f3s_preprocess_fill: tcbBitMap must be 8-byte aligned");
+  if (f3s::misaligned(tcbBitMap, 16) || f3s::misaligned(sparseAToXidx, 16))
+    return f3s::fail(-1, "f3s_preprocess_fill: tcbBitMap and sparseAToXidx must be 16-byte "
+                         "aligned (the attention kernels fetch them 16 bytes per lane)");
   return f3s::launch_preprocess_fill(rowPtr, colIdx, N, E, H, W, edgeToColumn, rowWindowOffset,
                                      nTCB, tcblockRowid, tcblocktileId, tcblockOffset,
                                      sparseAToXidx, tcbBitMap, static_cast<hipStream_t>(stream));
@@ -111,8 +112,9 @@ int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, i
     return f3s::fail(-1, "f3s_preprocess: null edge or block array");
   if (f3s::misaligned(workspace, 256))
     return f3s::fail(-1, "f3s_preprocess: workspace must be 256-byte aligned");
-  if (f3s::misaligned(tcbBitMap, 8))
-    return f3s::fail(-1, "f3s_preprocess: tcbBitMap must be 8-byte aligned");
+  if (f3s::misaligned(tcbBitMap, 16) || f3s::misaligned(sparseAToXidx, 16))
+    return f3s::fail(-1, "f3s_preprocess: tcbBitMap and sparseAToXidx must be 16-byte aligned "
+                         "(the attention kernels fetch them 16 bytes per lane)");
   return f3s::launch_preprocess(rowPtr, colIdx, N, E, H, W, blockPartition, edgeToColumn,
                                 edgeToRow, rowWindowOffset, sortedRowWindows, capacity,
                                 tcblockRowid, tcblocktileId, tcblockOffset, sparseAToXidx,
@@ -123,18 +125,45 @@ int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, i
 size_t f3s_attention_workspace_bytes(int N, int d) {
   if (N < 0) N = 0;
   if (d < 32) d = 32;
-  return f3s::attention_sliced_workspace_bytes(N, d);
+  return f3s::attention_sliced_workspace_bytes(N, d, 0);
+}
+
+size_t f3s_attention_heads_workspace_bytes(int N, int nHeads, int d) {
+  if (N < 0) N = 0;
+  if (d < 32) d = 32;
+  if (nHeads < 1) nHeads = 1;
+  return f3s::attention_sliced_workspace_bytes(N, d, nHeads);
 }
 
 int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype) {
   return f3s::attention_uses_workspace(N, nTCB, d, dtype);
 }
 
+int f3s_attention_uses_wide_offsets(int64_t N, int64_t pitch_bytes, int pitched) {
+  if (N < 0 || pitch_bytes < 0) return 0;
+  return f3s::gather_needs_wide_offsets(N, pitch_bytes, pitched != 0);
+}
+
+int f3s_attention_prepare(const int32_t* rowWindowOffset, const int32_t* sparseAToXidx, int N,
+                          int64_t nTCB, int d, int nHeads, void* workspace, size_t ws_bytes,
+                          void* stream) {
+  if (N <= 0 || nTCB < 0) return f3s::fail(-2, "f3s_attention_prepare: N must be positive");
+  if (!rowWindowOffset || !workspace || (nTCB > 0 && !sparseAToXidx))
+    return f3s::fail(-1, "f3s_attention_prepare: null pointer");
+  if (f3s::misaligned(workspace, 256) || f3s::misaligned(sparseAToXidx, 16))
+    return f3s::fail(-1, "f3s_attention_prepare: workspace needs 256-byte, sparseAToXidx 16-byte "
+                         "alignment");
+  return f3s::launch_attention_prepare(rowWindowOffset, sparseAToXidx, N, nTCB, d, nHeads,
+                                       workspace, ws_bytes,
+                                       static_cast<hipStream_t>(stream));
+}
+
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                       const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int64_t nTCB,
                       int d, int dtype, const void* Q, const void* K, const void* V,
                       float scalingFactor, int applySoftmax, float* out,
-                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, void* stream) {
+                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, int prepared,
+                      void* stream) {
   if (N < 0) return f3s::fail(-2, "f3s_attention_fwd: negative N");
   if (N == 0) return 0;
   if (!rowWindowOffset || !Q || !K || !V || !out)
@@ -147,18 +176,19 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
   if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd: negative nTCB");
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd: null TC-block arrays");
-  if (workspace && f3s::misaligned(workspace, 4))
-    return f3s::fail(-1, "f3s_attention_fwd: workspace must be 4-byte aligned");
+  if (workspace && f3s::misaligned(workspace, 256))
+    return f3s::fail(-1, "f3s_attention_fwd: workspace must be 256-byte aligned");
   return f3s::launch_attention(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N, nTCB, d,
                                dtype, Q, K, V, scalingFactor, applySoftmax, out, cuTimer,
-                               workspace, ws_bytes, static_cast<hipStream_t>(stream));
+                               workspace, ws_bytes, prepared, static_cast<hipStream_t>(stream));
 }
 
 int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                             const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
                             int64_t nTCB, int nHeads, int d, int dtype, const void* Q,
                             const void* K, const void* V, int64_t ldIn, float scalingFactor,
-                            int applySoftmax, float* out, int64_t ldOut, void* stream) {
+                            int applySoftmax, float* out, int64_t ldOut, void* workspace,
+                            size_t ws_bytes, int prepared, void* stream) {
   if (N < 0) return f3s::fail(-2, "f3s_attention_fwd_heads: negative N");
   if (N == 0) return 0;
   if (!rowWindowOffset || !Q || !K || !V || !out)
@@ -171,9 +201,12 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
   if (nTCB < 0) return f3s::fail(-2, "f3s_attention_fwd_heads: negative nTCB");
   if (nTCB > 0 && (!sparseAToXidx || !tcbBitMap))
     return f3s::fail(-1, "f3s_attention_fwd_heads: null TC-block arrays");
+  if (workspace && f3s::misaligned(workspace, 256))
+    return f3s::fail(-1, "f3s_attention_fwd_heads: workspace must be 256-byte aligned");
   return f3s::launch_attention_heads(rowWindowOffset, windowOrder, sparseAToXidx, tcbBitMap, N,
-                                     nTCB, nHeads, d, dtype, Q, K, V, ldIn, scalingFactor, applySoftmax,
-                                     out, ldOut, static_cast<hipStream_t>(stream));
+                                     nTCB, nHeads, d, dtype, Q, K, V, ldIn, scalingFactor,
+                                     applySoftmax, out, ldOut, workspace, ws_bytes, prepared,
+                                     static_cast<hipStream_t>(stream));
 }
 
 int f3s_attention_fwd_tcb8(const int32_t* rowWindowOffset, const int32_t* windowOrder,

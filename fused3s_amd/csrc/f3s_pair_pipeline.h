@@ -154,51 +154,105 @@ __device__ __forceinline__ void vm_wait() {
 }
 
 // ---- geometry of the per-wave LDS ring
+// D: head dimension, any multiple of 32 up to 256 (the reference takes embeddingDim at run time,
+// src/F3S_kernel.cu:601-604,1424,1522). The ring is laid out for DP, the next power of two: a row
+// of the LDS tile is DP elements wide, of which the first D hold data; lanes whose chunk does not
+// exist fetch nothing.
 template <int D>
 struct Geo {
-  static constexpr int T = D / 16;         // output tiles; gather instructions per 32-row tile
+  static_assert(D % 32 == 0 && D >= 32 && D <= 256, "head dimension: a multiple of 32 up to 256");
+  static constexpr int DP = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+  static constexpr int T = D / 16;         // output tiles
   static constexpr int KS = D / 32;        // k-steps of the score product
-  static constexpr int ROW = D * 2;        // bytes of a K / V row
-  static constexpr int CPR = D / 8;        // 16-byte chunks per row == lanes per gathered row
+  static constexpr int TG = DP / 16;       // gather instructions per 32-row tile
+  static constexpr int ROW = DP * 2;       // bytes of a K / V row in LDS
+  static constexpr int GROW = D * 2;       // bytes of a contiguous K / V row in memory
+  static constexpr int CHUNKS = D / 8;     // 16-byte chunks of a row that exist
+  static constexpr int CPR = DP / 8;       // 16-byte chunks per LDS row == lanes per gathered row
   static constexpr int RPI = 64 / CPR;     // rows per gather instruction
   static constexpr int TILE = 32 * ROW;    // K (or V) rows of one pair
   static constexpr int STAGE = 2 * TILE;   // one pair: K tile, then V tile
-  static constexpr int NS = D >= 128 ? 1 : 2;  // stages of the ring
+  static constexpr int NS = DP >= 128 ? 1 : 2;  // stages of the ring
   static constexpr int META_SLOT = 1024;   // metadata of four steps: 512 B ids, 256 B bitmaps
   static constexpr int META = 2 * META_SLOT;
   static constexpr int WAVE_BYTES = NS * STAGE + META;
 };
 
 // Which of the pair's 32 key slots lane-row rho of gather instruction i fetches, and its inverse
-// (the row of the LDS tile a slot lands in). Chosen so that the T slots a lane fetches are
-// consecutive dwords of the metadata (one LDS read yields all its row ids).
-template <int D>
+// (the row of the LDS tile a slot lands in: row i * RPI + rho). Chosen so that the slots a lane
+// fetches are groups of four consecutive dwords of the metadata (one 16-byte LDS read yields four
+// of its row ids). DP >= 64: slot = 4 * (rho + RPI * (i / 4)) + i % 4.
+template <int DP>
 __device__ __forceinline__ constexpr int slot_of(int i, int rho) {
-  if constexpr (D == 64) return 4 * rho + i;
-  if constexpr (D == 128) return 4 * (rho + 4 * (i >> 2)) + (i & 3);
-  return 4 * (rho >> 1) + 2 * i + (rho & 1);  // D == 32
+  if constexpr (DP == 32) return 4 * (rho >> 1) + 2 * i + (rho & 1);
+  constexpr int RPI = 512 / DP;
+  return 4 * (rho + RPI * (i >> 2)) + (i & 3);
 }
-template <int D>
+template <int DP>
 __device__ __forceinline__ constexpr int lds_row_of(int s) {
-  if constexpr (D == 64) return (s & 3) * 8 + (s >> 2);
-  if constexpr (D == 128) return ((s & 3) + 4 * (s >> 4)) * 4 + ((s >> 2) & 3);
-  return ((s & 3) >> 1) * 16 + 2 * (s >> 2) + (s & 1);  // D == 32
+  if constexpr (DP == 32) return ((s & 3) >> 1) * 16 + 2 * (s >> 2) + (s & 1);
+  constexpr int RPI = 512 / DP;
+  const int rho = (s >> 2) & (RPI - 1);
+  const int q = (s >> 2) / RPI;
+  return ((s & 3) + 4 * q) * RPI + rho;
 }
 // XOR applied to the 16-byte chunk index of slot s inside its LDS row: the K tile is read with
 // one 16-byte read per lane (16 consecutive slots by 4 chunks), the V tile with transposing
 // 8-byte reads (4 consecutive slots by 32 bytes); each pattern wants its rows on different banks.
-template <int D>
+template <int DP>
 __device__ __forceinline__ constexpr int swz_k(int s) {
   const int c = s & 15;
-  if constexpr (D == 64) return (c & 3) | ((((c >> 2) ^ (c >> 3)) & 1) << 2);
-  if constexpr (D == 128) return c;
-  return ((c >> 1) & 1) | ((((c >> 2) ^ (c >> 3)) & 1) << 1);  // D == 32
+  if constexpr (DP == 64) return (c & 3) | ((((c >> 2) ^ (c >> 3)) & 1) << 2);
+  if constexpr (DP >= 128) return c;
+  return ((c >> 1) & 1) | ((((c >> 2) ^ (c >> 3)) & 1) << 1);  // DP == 32
 }
-template <int D>
+template <int DP>
 __device__ __forceinline__ constexpr int swz_v(int s) {
-  if constexpr (D == 32) return ((s >> 1) & 1) << 1;
+  if constexpr (DP == 32) return ((s >> 1) & 1) << 1;
   return (s & 3) << 1;
 }
+// The chunk a lane fetches in gather instruction i depends on i only through i % NK (K) and
+// i % NV (V), so that many byte offsets are kept per lane.
+template <int DP>
+constexpr int distinct_k_offsets() {
+  return DP == 32 ? 2 : DP == 256 ? 8 : 4;
+}
+template <int DP>
+constexpr int distinct_v_offsets() {
+  return DP == 32 ? 2 : 4;
+}
+template <int DP>
+constexpr bool gather_offsets_periodic() {
+  constexpr int RPI = 512 / DP, TG = DP / 16;
+  for (int i = 0; i < TG; i++)
+    for (int rho = 0; rho < RPI; rho++) {
+      if (swz_k<DP>(slot_of<DP>(i, rho)) !=
+          swz_k<DP>(slot_of<DP>(i % distinct_k_offsets<DP>(), rho)))
+        return false;
+      if (swz_v<DP>(slot_of<DP>(i, rho)) !=
+          swz_v<DP>(slot_of<DP>(i % distinct_v_offsets<DP>(), rho)))
+        return false;
+    }
+  return true;
+}
+static_assert(gather_offsets_periodic<32>() && gather_offsets_periodic<64>() &&
+                  gather_offsets_periodic<128>() && gather_offsets_periodic<256>(),
+              "gather offsets must repeat with the stated periods");
+
+// the two maps are inverse to each other for every power-of-two width
+template <int DP>
+constexpr bool slot_maps_consistent() {
+  constexpr int RPI = 512 / DP, TG = DP / 16;
+  for (int i = 0; i < TG; i++)
+    for (int rho = 0; rho < RPI; rho++) {
+      const int s = slot_of<DP>(i, rho);
+      if (s < 0 || s >= 32 || lds_row_of<DP>(s) != i * RPI + rho) return false;
+    }
+  return true;
+}
+static_assert(slot_maps_consistent<32>() && slot_maps_consistent<64>() &&
+                  slot_maps_consistent<128>() && slot_maps_consistent<256>(),
+              "slot_of and lds_row_of must be inverse");
 
 // Problem description shared by every kernel.
 template <typename ET>
@@ -217,14 +271,21 @@ struct Problem {
 
 // ET: _Float16 or __bf16. HEADS: pitched rows (row offset by 24-bit multiply). W8: the structure
 // comes from preprocessing with 8-column blocks; two consecutive 16x8 blocks are laid out like
-// one 16x16 block, block indices and counts below are then in 16x8 blocks.
-template <typename ET, int D, bool SOFTMAX, bool HEADS, bool W8>
+// one 16x16 block, block indices and counts below are then in 16x8 blocks. WIDE: K or V spans
+// 4 GiB or more (or a pitched layout exceeds the 24-bit multiply): row offsets in 64 bits.
+template <typename ET, int D, bool SOFTMAX, bool HEADS, bool W8, bool WIDE = false>
 struct PairPipeline {
   typedef Geo<D> G;
   typedef typename Vec<ET, 8>::type half8;
   static constexpr int T = G::T;
   static constexpr int KS = G::KS;
   static constexpr int NS = G::NS;
+  static constexpr int TG = G::TG;
+  static constexpr int DP = G::DP;
+  static constexpr int NK = distinct_k_offsets<DP>();
+  static constexpr int NV = distinct_v_offsets<DP>();
+  static constexpr int NVA = T < 4 ? T : 4;  // V read addresses kept: tile j reads at
+                                             // vReadAddr[j % 4] + (j / 4) * 128
   static constexpr int BPS = W8 ? 4 : 2;  // blocks of the structure per step
   static constexpr bool SPLIT_P = sizeof(ET) == 2 && !__is_same(ET, _Float16);  // bf16
 
@@ -237,11 +298,12 @@ struct PairPipeline {
   unsigned ring;        // LDS byte address of this wave's ring
   unsigned metaBase;    // LDS byte address of this wave's two metadata slots
   unsigned kReadAddr[2][KS];  // K tile: slot 16b + c, chunk 4i + g (swizzled)
-  unsigned vReadAddr[T];   // V tile: transposing read of tile j, first key half
+  unsigned vReadAddr[NVA];  // V tile: transposing read of tiles 0..3, first key half
   unsigned idReadAddr;     // metadata: this lane's row ids
   unsigned maskReadAddr;   // metadata: the bitmap dword with this lane's bits of block A
   int keepPos[4];          // bit position of element i in that dword
-  uint32_t gatherOffK[T], gatherOffV[T];  // byte offset inside the row this lane fetches
+  uint32_t gatherOffK[NK], gatherOffV[NV];  // byte offset inside the row this lane fetches
+  uint32_t gatherLive;  // D < DP: bit i / bit 16 + i: the chunk of K / V instruction i exists
   int lane, g, c;
 
   __device__ __forceinline__ void init(const Problem<ET>& pb, int w, unsigned ringAddr, int head) {
@@ -271,11 +333,15 @@ struct PairPipeline {
     // slot_of(i, lane / CPR); the chunk lands at ring + i * 1024 + lane * 16
     const int rho = lane / G::CPR;
     const int pos = lane % G::CPR;
+    gatherLive = 0;
 #pragma unroll
-    for (int i = 0; i < T; i++) {
-      const int s = slot_of<D>(i, rho);
-      gatherOffK[i] = (uint32_t)((pos ^ swz_k<D>(s)) * 16 + (HEADS ? head * D * 2 : 0));
-      gatherOffV[i] = (uint32_t)((pos ^ swz_v<D>(s)) * 16 + (HEADS ? head * D * 2 : 0));
+    for (int i = 0; i < TG; i++) {
+      const int s = slot_of<DP>(i, rho);
+      const int ck = pos ^ swz_k<DP>(s), cv = pos ^ swz_v<DP>(s);
+      if (i < NK) gatherOffK[i] = (uint32_t)(ck * 16 + (HEADS ? head * D * 2 : 0));
+      if (i < NV) gatherOffV[i] = (uint32_t)(cv * 16 + (HEADS ? head * D * 2 : 0));
+      if (ck < G::CHUNKS) gatherLive |= 1u << i;
+      if (cv < G::CHUNKS) gatherLive |= 1u << (16 + i);
     }
     // score product: lane (g, c) reads, for block b and k-step i, chunk 4i + g of slot 16b + c
 #pragma unroll
@@ -283,7 +349,7 @@ struct PairPipeline {
       const int s = 16 * b + c;
 #pragma unroll
       for (int i = 0; i < KS; i++)
-        kReadAddr[b][i] = ring + lds_row_of<D>(s) * G::ROW + (((4 * i + g) ^ swz_k<D>(s)) * 16);
+        kReadAddr[b][i] = ring + lds_row_of<DP>(s) * G::ROW + (((4 * i + g) ^ swz_k<DP>(s)) * 16);
     }
     // P V product: lane (g, c = 4e + x) addresses slot 16h + 4g + e, columns 16j + 4x .. +3:
     // chunk 2j + x/2 (swizzled), byte (x % 2) * 8 inside it. h = 1 is a fixed distance away.
@@ -291,12 +357,12 @@ struct PairPipeline {
       const int e = c >> 2, x = c & 3;
       const int s = 4 * g + e;
 #pragma unroll
-      for (int j = 0; j < T; j++)
-        vReadAddr[j] = ring + G::TILE + lds_row_of<D>(s) * G::ROW +
-                       (((2 * j + (x >> 1)) ^ swz_v<D>(s)) * 16) + (x & 1) * 8;
+      for (int j = 0; j < NVA; j++)
+        vReadAddr[j] = ring + G::TILE + lds_row_of<DP>(s) * G::ROW +
+                       (((2 * j + (x >> 1)) ^ swz_v<DP>(s)) * 16) + (x & 1) * 8;
     }
     // metadata slot: ids of step q at q * 128, bitmaps at 512 + q * 64
-    if constexpr (D == 32)
+    if constexpr (DP == 32)
       idReadAddr = metaBase + (4 * (rho >> 1) + (rho & 1)) * 4;
     else
       idReadAddr = metaBase + rho * 16;
@@ -335,53 +401,75 @@ struct PairPipeline {
   // K and V rows of step p into ring stage `stage` (compile-time), row ids from metadata.
   template <int STAGE_IDX, int Q4>
   __device__ __forceinline__ void issue_gather(const Problem<ET>& pb, int metaSlot) {
-    // row ids of this lane's T slots: consecutive dwords of the step's 32 ids
-    int rows[T];
+    // row ids of this lane's TG slots: groups of four consecutive dwords of the step's 32 ids
+    int rows[TG];
     const unsigned ida = idReadAddr + metaSlot * G::META_SLOT;
-    if constexpr (D == 64) {
-      const int4v r = lds_read_b128<Q4 * 128>(ida);
-      lds_wait();
-#pragma unroll
-      for (int i = 0; i < 4; i++) rows[i] = r[i];
-    } else if constexpr (D == 128) {
-      const int4v r0 = lds_read_b128<Q4 * 128>(ida);
-      const int4v r1 = lds_read_b128<Q4 * 128 + 64>(ida);
-      lds_wait();
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        rows[i] = r0[i];
-        rows[4 + i] = r1[i];
-      }
-    } else {
+    if constexpr (DP == 32) {
       const int2v r = lds_read2_b32<Q4 * 32, Q4 * 32 + 2>(ida);
       lds_wait();
       rows[0] = r[0];
       rows[1] = r[1];
+    } else {
+      // group q of four slots starts RPI * 4 slots (RPI * 16 bytes) after group q - 1
+      int4v r[TG / 4];
+      r[0] = lds_read_b128<Q4 * 128>(ida);
+      if constexpr (TG >= 8) r[1] = lds_read_b128<Q4 * 128 + 1 * G::RPI * 16>(ida);
+      if constexpr (TG >= 16) {
+        r[2] = lds_read_b128<Q4 * 128 + 2 * G::RPI * 16>(ida);
+        r[3] = lds_read_b128<Q4 * 128 + 3 * G::RPI * 16>(ida);
+      }
+      lds_wait();
+#pragma unroll
+      for (int q = 0; q < TG / 4; q++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) rows[4 * q + i] = r[q][i];
     }
     const char* Kb = reinterpret_cast<const char*>(pb.K);
     const char* Vb = reinterpret_cast<const char*>(pb.V);
-    const uint32_t rowBytes = (uint32_t)pb.pitchIn * 2u;
+    const uint32_t rowBytes = HEADS ? (uint32_t)pb.pitchIn * 2u : (uint32_t)G::GROW;
     const int ringU = uniform((int)ring);
 #pragma unroll
-    for (int i = 0; i < T; i++) {
+    for (int i = 0; i < TG; i++) {
       pin(rows[i]);
 #ifdef F3S_PROBE_ROWMASK
       rows[i] &= F3S_PROBE_ROWMASK;
 #endif
-      const uint32_t ro = HEADS ? __umul24((uint32_t)rows[i], rowBytes)
-                                : (uint32_t)rows[i] * (uint32_t)G::ROW;
-      const uint32_t ko = ro + gatherOffK[i];
-      F3S_LDS int4v* dst = (F3S_LDS int4v*)(uintptr_t)(ringU + STAGE_IDX * G::STAGE + i * 1024);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4v*>(Kb + ko), dst, 16, 0, 0);
     }
+    // one gather instruction: 64 lanes x 16 bytes of K (V) rows into 1 KiB of the stage
+    auto gather = [&](const char* src, bool live, int ldsOffset) {
+      F3S_LDS int4v* dst = (F3S_LDS int4v*)(uintptr_t)(ringU + ldsOffset);
+      if constexpr (D == DP) {
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4v*>(src), dst, 16, 0, 0);
+      } else {
+        if (live)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4v*>(src), dst, 16, 0, 0);
+      }
+    };
+    if constexpr (WIDE) {
+      // the reference indexes rows with int64_t (src/F3S_kernel.cu:1422-1423)
 #pragma unroll
-    for (int i = 0; i < T; i++) {
-      const uint32_t ro = HEADS ? __umul24((uint32_t)rows[i], rowBytes)
-                                : (uint32_t)rows[i] * (uint32_t)G::ROW;
-      const uint32_t vo = ro + gatherOffV[i];
-      F3S_LDS int4v* dst =
-          (F3S_LDS int4v*)(uintptr_t)(ringU + STAGE_IDX * G::STAGE + G::TILE + i * 1024);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const int4v*>(Vb + vo), dst, 16, 0, 0);
+      for (int i = 0; i < TG; i++)
+        gather(Kb + ((uint64_t)(uint32_t)rows[i] * rowBytes + gatherOffK[i % NK]),
+               (gatherLive >> i) & 1u, STAGE_IDX * G::STAGE + i * 1024);
+#pragma unroll
+      for (int i = 0; i < TG; i++)
+        gather(Vb + ((uint64_t)(uint32_t)rows[i] * rowBytes + gatherOffV[i % NV]),
+               (gatherLive >> (16 + i)) & 1u, STAGE_IDX * G::STAGE + G::TILE + i * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < TG; i++) {
+        const uint32_t ro = HEADS ? __umul24((uint32_t)rows[i], rowBytes)
+                                  : (uint32_t)rows[i] * rowBytes;
+        gather(Kb + (ro + gatherOffK[i % NK]), (gatherLive >> i) & 1u,
+               STAGE_IDX * G::STAGE + i * 1024);
+      }
+#pragma unroll
+      for (int i = 0; i < TG; i++) {
+        const uint32_t ro = HEADS ? __umul24((uint32_t)rows[i], rowBytes)
+                                  : (uint32_t)rows[i] * rowBytes;
+        gather(Vb + (ro + gatherOffV[i % NV]), (gatherLive >> (16 + i)) & 1u,
+               STAGE_IDX * G::STAGE + G::TILE + i * 1024);
+      }
     }
   }
 
@@ -399,16 +487,20 @@ struct PairPipeline {
     for (int b = 0; b < 2; b++)
 #pragma unroll
       for (int i = 0; i < KS; i++) op.k[b][i] = lds_read_b128<SO>(kReadAddr[b][i]);
-#pragma unroll
-    for (int j = 0; j < T; j++) {
-      op.v[j][0] = lds_read_tr16_b64<SO>(vReadAddr[j]);
-      op.v[j][1] = lds_read_tr16_b64<SO + v_half_distance()>(vReadAddr[j]);
-    }
+    read_v_tile<SO, 0>(op);
     op.words = lds_read2_b32<Q4 * 16, Q4 * 16 + 8>(maskReadAddr + metaSlot * G::META_SLOT);
+  }
+  // tile J of the V operand: 128 bytes (eight chunks) per four tiles beyond tile J % 4
+  template <int SO, int J>
+  __device__ __forceinline__ void read_v_tile(Operands& op) {
+    constexpr int OFF = SO + (J / 4) * 128;
+    op.v[J][0] = lds_read_tr16_b64<OFF>(vReadAddr[J % 4]);
+    op.v[J][1] = lds_read_tr16_b64<OFF + v_half_distance()>(vReadAddr[J % 4]);
+    if constexpr (J + 1 < T) read_v_tile<SO, J + 1>(op);
   }
   // LDS distance between the rows of slot s and slot s + 16 of a tile
   static __device__ __forceinline__ constexpr int v_half_distance() {
-    return (lds_row_of<D>(16) - lds_row_of<D>(0)) * G::ROW;
+    return (lds_row_of<DP>(16) - lds_row_of<DP>(0)) * G::ROW;
   }
 
   __device__ __forceinline__ void consume(Operands& op) {
@@ -577,7 +669,7 @@ struct PairPipeline {
        steps opened a group of four, its metadata load */                                     \
     if constexpr (NS == 2) {                                                                   \
       if (p + 1 < nSteps) {                                                                    \
-        if (Q4 == 1 && metaIssued) vm_wait<2 * T + 1>(); else vm_wait<2 * T>();                \
+        if (Q4 == 1 && metaIssued) vm_wait<2 * TG + 1>(); else vm_wait<2 * TG>();                \
       } else {                                                                                 \
         vm_wait<0>();                                                                          \
       }                                                                                        \

@@ -196,6 +196,38 @@ struct Launch {
   const char* timerFile;  // non-null: record per-CU active time into this file
 };
 
+// Scratch of the column-sliced schedule: one tensor per device, kept between calls and grown when
+// a call needs more. A call holds the lock from the moment it takes the tensor until its kernels
+// are done (every entry point blocks on its stop event, see timed_launch), so two host threads
+// never compute into the same scratch. F3S.release_workspace() drops the tensors.
+std::mutex g_wsMutex;
+std::map<int, torch::Tensor> g_wsCache;
+
+struct WorkspaceLease {
+  std::unique_lock<std::mutex> lock;
+  torch::Tensor tensor;
+  WorkspaceLease(bool wanted, size_t bytes, const c10::Device& device) {
+    if (!wanted) return;
+    lock = std::unique_lock<std::mutex>(g_wsMutex);
+    torch::Tensor& cached = g_wsCache[(int)device.index()];
+    if (!cached.defined() || (size_t)cached.numel() < bytes)
+      cached = torch::empty({(int64_t)bytes},
+                            torch::TensorOptions().dtype(torch::kUInt8).device(device));
+    tensor = cached;
+  }
+};
+
+// F3S.release_workspace(): frees the cached scratch of every device (beyond the reference's
+// surface, whose launchers keep nothing between calls). Returns the number of bytes released.
+int64_t releaseWorkspace() {
+  std::lock_guard<std::mutex> lock(g_wsMutex);
+  int64_t bytes = 0;
+  for (auto& kv : g_wsCache)
+    if (kv.second.defined()) bytes += kv.second.numel();
+  g_wsCache.clear();
+  return bytes;
+}
+
 // Common host path of every 1tb1rw entry point: f3sCuda1tb1rw / f3sCuda1tb1rwScheduled and the
 // Clocked launchers (src/F3S_kernel.cu:393-671). Returns {time_ms (0-d CPU fp32), out fp32[N,d],
 // empty fp32 sddmmResult} like the reference. `out` is allocated [N, d] (the reference
@@ -247,25 +279,15 @@ std::vector<torch::Tensor> run_1tb1rw(const torch::Tensor& rowWindowOffset,
   const bool sliced = !L.timerFile && f3s_attention_uses_workspace(
                                           nNodes, sparseAToXidx.numel() / 16, (int)d, dtype) != 0;
   const size_t wsBytes = sliced ? f3s_attention_workspace_bytes(nNodes, (int)d) : 0;
-  // one scratch tensor per device, kept between calls and grown when a call needs more; every
-  // entry point blocks until its kernels are done (see timed_launch), so calls cannot overlap
-  static std::mutex wsMutex;
-  static std::map<int, torch::Tensor> wsCache;
-  torch::Tensor workspace;
-  if (sliced) {
-    std::lock_guard<std::mutex> lock(wsMutex);
-    torch::Tensor& cached = wsCache[(int)Q.device().index()];
-    if (!cached.defined() || (size_t)cached.numel() < wsBytes)
-      cached = torch::empty({(int64_t)wsBytes}, f32.dtype(torch::kUInt8));
-    workspace = cached;
-  }
+  WorkspaceLease lease(sliced, wsBytes, Q.device());
+  torch::Tensor& workspace = lease.tensor;
   const float ms = timed_launch("f3s_attention_fwd", [&](void* stream) {
     return f3s_attention_fwd(
         rowWindowOffset.data_ptr<int>(), L.order ? L.order->data_ptr<int>() : nullptr,
         sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
         nNodes, sparseAToXidx.numel() / 16, (int)d, dtype, Q.data_ptr(), K.data_ptr(),
         V.data_ptr(), L.scalingFactor, L.applySoftmax ? 1 : 0, out.data_ptr<float>(), timerPtr,
-        sliced ? workspace.data_ptr() : nullptr, wsBytes, stream);
+        sliced ? workspace.data_ptr() : nullptr, wsBytes, 0, stream);
   });
   if (L.timerFile) write_cu_time(timer, nRW, L.timerFile);
   auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));
@@ -306,13 +328,19 @@ std::vector<torch::Tensor> f3sMultiHeadScaleQK(torch::Tensor rowWindowOffset,
   auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(Q.device());
   auto out = torch::empty({(int64_t)nNodes, nHeads * d}, f32);
   const int dtype = Q.scalar_type() == torch::kHalf ? F3S_DTYPE_F16 : F3S_DTYPE_BF16;
+  // graphs of long windows take the column-sliced schedule here as in the single-head calls
+  const bool sliced =
+      f3s_attention_uses_workspace(nNodes, sparseAToXidx.numel() / 16, (int)d, dtype) != 0;
+  const size_t wsBytes =
+      sliced ? f3s_attention_heads_workspace_bytes(nNodes, (int)nHeads, (int)d) : 0;
+  WorkspaceLease lease(sliced, wsBytes, Q.device());
   const float ms = timed_launch("f3s_attention_fwd_heads", [&](void* stream) {
     return f3s_attention_fwd_heads(
         rowWindowOffset.data_ptr<int>(), sortedRowWindows.data_ptr<int>(),
         sparseAToXidx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(tcbBitMap.data_ptr()),
         nNodes, sparseAToXidx.numel() / 16, (int)nHeads, (int)d, dtype, Q.data_ptr(),
         K.data_ptr(), V.data_ptr(), Q.stride(0), scalingFactor, 1, out.data_ptr<float>(),
-        out.stride(0), stream);
+        out.stride(0), sliced ? lease.tensor.data_ptr() : nullptr, wsBytes, 0, stream);
   });
   auto time = torch::tensor(ms, torch::TensorOptions().dtype(torch::kFloat32));
   return {time, out, torch::zeros({0}, f32)};
@@ -424,4 +452,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "fused3S 1tb1rw scheduled permuteV scaleQK");
   m.def("f3s_multihead_scaleQK", &f3sMultiHeadScaleQK,
         "fused3S over [N, heads, d] Q/K/V in one launch (fp16 or bf16), heavy-first order");
+  m.def("release_workspace", &releaseWorkspace,
+        "free the cached scratch of the column-sliced schedule; returns the bytes released");
 }

@@ -99,6 +99,8 @@ int f3s_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, in
  *   sparseAToXidx  [nTCB*W]        out: original column of each compacted slot, 0 when unused
  *   tcbBitMap      [nTCB*H*W/64] (uint64)  out: 8x8 sub-blocks in column-major order,
  *                                  row-major and MSB-first inside a sub-block
+ * sparseAToXidx and tcbBitMap must be 16-byte aligned (here and in f3s_preprocess), as the
+ * attention entry points require of them.
  * Asynchronous on `stream`. Outputs are fully written.
  */
 int f3s_preprocess_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H, int W,
@@ -144,13 +146,16 @@ int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, i
  *   rowWindowOffset [nRW+1], sparseAToXidx [nTCB*16], tcbBitMap [nTCB*4]   from preprocessing
  *   windowOrder [nRW] or NULL      launch order of the row windows: sortedRowWindows for the
  *                                  heavy-first schedule, NULL for natural order
- *   N, nTCB, d                     nodes; TC blocks (rowWindowOffset[nRW]); head dimension
- *                                  (32, 64 or 128)
+ *   N, nTCB, d                     nodes; TC blocks (rowWindowOffset[nRW]); head dimension: a
+ *                                  multiple of 32 up to 256 (the reference takes embeddingDim
+ *                                  at run time, src/F3S_kernel.cu:601-604,1424,1522)
  *   dtype                          F3S_DTYPE_F16 (the reference's only type) or F3S_DTYPE_BF16
  *                                  (bf16 MFMA; the probabilities then enter the second product as
  *                                  the sum of two bf16 terms, 16 bits of mantissa instead of the
  *                                  11 of the reference's fp16 rounding)
- *   Q, K, V [N*d]                  row-major, contiguous
+ *   Q, K, V [N*d]                  row-major, contiguous; any size (row offsets are formed in
+ *                                  64 bits once an array reaches 4 GiB, as the reference's
+ *                                  int64_t offsets are, src/F3S_kernel.cu:1422-1423)
  *   scalingFactor                  unmasked scores are DIVIDED by it (src/F3S_kernel.cu:1666-1667);
  *                                  1.0 = unscaled (:612-613)
  *   applySoftmax                   0 = SDDMM -> SpMM only (src/F3S_kernel.cu:420-443)
@@ -158,34 +163,65 @@ int f3s_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, i
  *   cuTimer                        NULL, or 3*nRW uint64 {begin, end, cu id} per workgroup
  *                                  (the Clocked variants, src/F3S_kernel.cu:1178-1368, 1803-1997)
  *   workspace, ws_bytes            NULL / 0, or device scratch of
- *                                  f3s_attention_workspace_bytes(N, d) bytes (4-byte aligned).
+ *                                  f3s_attention_workspace_bytes(N, d) bytes (256-byte aligned).
  *                                  With it, graphs for which f3s_attention_uses_workspace()
  *                                  returns 1 are computed by the column-sliced schedule: per
  *                                  (window, column slice) partial results that a second kernel
- *                                  merges. Results agree with the default schedule within the
- *                                  tolerance of the summation order. Ignored with cuTimer.
- * Asynchronous on `stream`.
+ *                                  merges in slice order. Results agree with the default
+ *                                  schedule within the tolerance of the summation order.
+ *                                  Ignored with cuTimer. Calls that share a workspace must not
+ *                                  overlap. Its contents need not be initialised.
+ *   prepared                       0, or 1 when f3s_attention_prepare was called on this workspace
+ *                                  for these arrays: the schedule's index is then not rebuilt
+ *                                  (the call checks on the device that the workspace's header
+ *                                  names these arrays and rebuilds the index otherwise)
+ * Asynchronous on `stream` (kernel launches only: no host wait, no copy, no allocation).
  */
 int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                       const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N, int64_t nTCB,
                       int d, int dtype, const void* Q, const void* K, const void* V,
                       float scalingFactor, int applySoftmax, float* out,
-                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, void* stream);
+                      unsigned long long* cuTimer, void* workspace, size_t ws_bytes, int prepared,
+                      void* stream);
 
 /*
- * Bytes of device scratch f3s_attention_fwd can use for a graph of N nodes at head dimension d
- * (slice boundaries per window, 256 bytes of queue cursors, plus one partial (m, l, O) per window
- * and slice: about 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers
- * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
+ * Bytes of device scratch f3s_attention_fwd / f3s_attention_fwd_heads can use for a graph of N
+ * nodes at head dimension d (a header, the slice boundaries of every window, plus one partial
+ * (m, l, O) per window, head and slice: about 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers (src/F3S_kernel.cu:581-671) need no scratch;
+ * passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);
+size_t f3s_attention_heads_workspace_bytes(int N, int nHeads, int d);
+
+/*
+ * Optional: builds the part of the column-sliced schedule that depends only on the TC-block
+ * structure (the slice boundaries of every window) in `workspace` once, so that the attention
+ * calls that follow (with prepared = 1) do not rebuild it. It has no counterpart in the reference
+ * (whose launchers keep no state between calls). The workspace then belongs to exactly these
+ * arrays (rowWindowOffset, sparseAToXidx: same pointers, same N, nTCB, d and head count; nHeads =
+ * 0 for f3s_attention_fwd, the head count for f3s_attention_fwd_heads): the caller must not
+ * change their contents, nor write to the workspace, while it passes prepared = 1. A call with
+ * prepared = 0, or with other arrays, on the same workspace rebuilds the index and ends the
+ * preparation. Asynchronous on `stream`.
+ */
+int f3s_attention_prepare(const int32_t* rowWindowOffset, const int32_t* sparseAToXidx, int N,
+                          int64_t nTCB, int d, int nHeads, void* workspace, size_t ws_bytes,
+                          void* stream);
 
 /*
  * 1 if f3s_attention_fwd would use a workspace for this problem (at least 2048 row windows with
  * 64 or more TC blocks each on average), else 0: callers can skip the allocation.
- * F3S_SCHEDULE=window or =sliced in the environment forces 0 or 1.
+ * F3S_SCHEDULE=window or =sliced in the environment (read at every call) forces 0 or 1.
  */
 int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype);
+
+/*
+ * 1 if the attention kernels form 64-bit row offsets for K / V arrays of N rows with a row pitch
+ * of pitch_bytes (pitched = 1: the multi-head layout): the array spans 4 GiB or more, or, with
+ * pitched rows, N or the pitch reaches 2^24. Informational; the entry points decide by
+ * themselves. The reference always uses int64_t offsets (src/F3S_kernel.cu:1422-1423).
+ */
+int f3s_attention_uses_wide_offsets(int64_t N, int64_t pitch_bytes, int pitched);
 
 /*
  * The same fused kernel over nHeads attention heads in one launch: Q, K, V are [N, nHeads, d]
@@ -194,14 +230,18 @@ int f3s_attention_uses_workspace(int N, int64_t nTCB, int d, int dtype);
  * concatenated. All heads share one graph (one TC-block structure). The reference has no
  * multi-head entry: its callers run f3s_1tb1rw_scheduled_permuteV_scaleQK (src/F3S.cpp:247-270)
  * once per head on contiguous per-head copies and concatenate; this call returns what that loop
- * returns. ldIn % 8 == 0, ldOut % 4 == 0, N < 2^24, ldIn*2 < 2^24, N*ldIn*2 < 2^32.
- * Asynchronous on `stream`.
+ * returns. ldIn % 8 == 0, ldOut % 4 == 0, both below 2^31.
+ * workspace, ws_bytes: NULL / 0, or f3s_attention_heads_workspace_bytes(N, nHeads, d) bytes of
+ * device scratch (256-byte aligned); with it, graphs for which f3s_attention_uses_workspace()
+ * returns 1 take the column-sliced schedule with (window, slice, head) units, as in
+ * f3s_attention_fwd; prepared as there. Asynchronous on `stream`.
  */
 int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windowOrder,
                             const int32_t* sparseAToXidx, const uint64_t* tcbBitMap, int N,
                             int64_t nTCB, int nHeads, int d, int dtype, const void* Q,
                             const void* K, const void* V, int64_t ldIn, float scalingFactor,
-                            int applySoftmax, float* out, int64_t ldOut, void* stream);
+                            int applySoftmax, float* out, int64_t ldOut, void* workspace,
+                            size_t ws_bytes, int prepared, void* stream);
 
 /*
  * Fused SDDMM -> softmax -> SpMM over 16x8 TC blocks: replaces f3sCuda1tb1tcb and
@@ -211,7 +251,7 @@ int f3s_attention_fwd_heads(const int32_t* rowWindowOffset, const int32_t* windo
  *   rowWindowOffset [nRW+1], sparseAToXidx [nTCB*8], tcbBitMap [nTCB*2]   from preprocessing
  *                                  with H = 16, W = 8
  *   windowOrder [nRW] or NULL      launch order (the reference launches in natural order)
- *   Q, K, V [N*d]                  fp16, row-major, contiguous; d in {32, 64, 128}
+ *   Q, K, V [N*d]                  fp16, row-major, contiguous; d a multiple of 32 up to 256
  *   applySoftmax                   0 = SDDMM -> SpMM only; scores are never scaled on this path
  *   out [N*d] float                fully written
  *   sddmmResult                    NULL, or nTCB*128 floats: the masked scores of every block,

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert getattr(lib, n) is not None
     lib.f3s_abi_version.restype = ctypes.c_int
-    assert lib.f3s_abi_version() == 1
+    assert lib.f3s_abi_version() == 2
     lib.f3s_last_error.restype = ctypes.c_char_p
     assert isinstance(lib.f3s_last_error(), bytes)
     lib.f3s_preprocess_workspace_bytes.restype = ctypes.c_size_t
@@ -38,10 +38,10 @@ def test_argument_errors_are_statuses_not_exits():
     from fused3s_amd import capi
     L = capi.lib()
     rc = L.f3s_attention_fwd(None, None, None, None, -1, 0, 64, 0, None, None, None, 1.0, 1, None,
-                             None, None, 0, None)
+                             None, None, 0, 0, None)
     assert rc != 0 and b"negative" in L.f3s_last_error()
     rc = L.f3s_attention_fwd(None, None, None, None, 5, 0, 64, 0, None, None, None, 1.0, 1, None,
-                             None, None, 0, None)
+                             None, None, 0, 0, None)
     assert rc != 0 and b"null" in L.f3s_last_error()
     n = ctypes.c_int64(0)
     rc = L.f3s_preprocess_count(None, None, 5, 0, 16, 16, None, None, None, None, None, None, 0,
