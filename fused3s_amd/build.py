@@ -31,6 +31,9 @@ HIP_FLAGS = [
 # fused3s_amd/probes/libf3s_amd_<name>.so and is used by pointing F3S_AMD_LIB at it, e.g.
 #     F3S_AMD_LIB=fused3s_amd/probes/libf3s_amd_gather_only.so python bench.py --no-cpu-baseline
 PROBES = {
+    # the column-sliced schedule's partial results through the caches instead of past them
+    "partial_cached_load": ["-DF3S_PROBE_PARTIAL_CACHED_LOAD"],
+    "partial_cached": ["-DF3S_PROBE_PARTIAL_CACHED_LOAD", "-DF3S_PROBE_PARTIAL_CACHED_STORE"],
     # K/V rows and metadata are gathered into LDS, nothing reads them back, no arithmetic
     "gather_only": ["-DF3S_PROBE_NO_COMPUTE", "-DF3S_PROBE_NO_READ"],
     # the same with every gathered row taken from the first 16384 rows (2 MiB of K, 2 MiB of V:

@@ -73,14 +73,26 @@ __device__ __forceinline__ pipe::Problem<ET> make_problem(const int32_t* sparseA
   return pb;
 }
 
+// probe builds: the partials through the caches instead of past them
+#ifdef F3S_PROBE_PARTIAL_CACHED_STORE
+#define F3S_PARTIAL_STORE(v, p) (*(p) = (v))
+#else
+#define F3S_PARTIAL_STORE(v, p) __builtin_nontemporal_store((v), (p))
+#endif
+#ifdef F3S_PROBE_PARTIAL_CACHED_LOAD
+#define F3S_PARTIAL_LOAD(p) (*(p))
+#else
+#define F3S_PARTIAL_LOAD(p) __builtin_nontemporal_load(p)
+#endif
+
 template <int D, typename PipeT>
 __device__ __forceinline__ void store_partial(const PipeT& pp, float* __restrict__ dst) {
 #pragma unroll
   for (int jj = 0; jj < D / 16; jj++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) __builtin_nontemporal_store(pp.o[jj][i], dst + (jj * 4 + i) * 64);
-  __builtin_nontemporal_store(pp.m, dst + (D / 4) * 64);
-  __builtin_nontemporal_store(pp.l, dst + (D / 4 + 1) * 64);
+    for (int i = 0; i < 4; i++) F3S_PARTIAL_STORE(pp.o[jj][i], dst + (jj * 4 + i) * 64);
+  F3S_PARTIAL_STORE(pp.m, dst + (D / 4) * 64);
+  F3S_PARTIAL_STORE(pp.l, dst + (D / 4 + 1) * 64);
 }
 
 // One wave per unit, kUnitWaves independent units per workgroup. A unit is
@@ -400,7 +412,7 @@ __global__ __launch_bounds__(256) void f3s_merge_slices_kernel(
           const float* src = base + (int64_t)sel[k] * partial_dwords<D>();
 #pragma unroll
           for (int r = 0; r < R + (SOFTMAX ? 2 : 0); r++)
-            v[k][r] = __builtin_nontemporal_load(src + r * 64);
+            v[k][r] = F3S_PARTIAL_LOAD(src + r * 64);
         }
       }
 #pragma unroll

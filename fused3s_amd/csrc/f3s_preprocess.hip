@@ -31,7 +31,6 @@
 //                        in CSR order (src/utils.cu:173-224, 23-36, 53-65).
 //
 // All results are bit-identical to the reference's algorithm with edgeToRow[e] = row(e).
-#include <hipcub/hipcub.hpp>
 
 #include <mutex>
 
@@ -484,9 +483,12 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
 }
 
 // Windows of kSortMax < edges <= kMedMax on graphs whose column range needs several bitset passes
-// (N > kRangeMax): one workgroup per queued window sorts the window's column ids (block-wide
-// radix sort), compacts the distinct ones and ranks every edge by binary search, instead of
-// several passes over a 48 KiB bitset that such a window fills with a few thousand bits.
+// (N > kRangeMax): one workgroup per queued window sorts the window's column ids, compacts the
+// distinct ones and ranks every edge by binary search, instead of several passes over a 48 KiB
+// bitset that such a window fills with a few thousand bits. The sort is the wave-level LSD radix
+// sort of window_rank_radix_kernel widened to a workgroup: eight bits per pass, every wave on its
+// own contiguous quarter of the keys (histogram with LDS atomics, one thread per digit turns the
+// per-wave counts into start positions, in-order scatter with wave ballots), two LDS buffers.
 constexpr int kMedThreads = 256;
 constexpr int kMedItems = 16;
 constexpr int kMedMax = kMedThreads * kMedItems;
@@ -497,18 +499,17 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
     int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
     int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
     const int32_t* __restrict__ bigList) {
-  typedef hipcub::BlockRadixSort<unsigned, kMedThreads, kMedItems> Sort;
-  __shared__ union {
-    typename Sort::TempStorage sort;
-    unsigned keys[kMedMax];
-  } u;
-  __shared__ unsigned sUniq[kMedMax];
+  constexpr int WAVES = kMedThreads / 64;
+  static_assert(kMedThreads == 256, "one thread per 8-bit digit");
+  __shared__ uint32_t sBuf[2][kMedMax];
+  __shared__ uint32_t sHist[WAVES][256];
   __shared__ int sRow[17];
-  __shared__ unsigned sWaveTot[kMedThreads / 64];
+  __shared__ unsigned sWaveTot[WAVES];
   __shared__ int sTake;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const unsigned long long ltMask = (1ull << lane) - 1ull;
   const int nBig = hdr->nBig;
   while (true) {
     __syncthreads();
@@ -522,35 +523,80 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
     const int eS = sRow[0], eE = sRow[16];
     const int n = eE - eS;
     if (n > kMedMax) continue;  // left to window_rank_kernel
-    unsigned keys[kMedItems];
     bool bad = false;
-#pragma unroll
-    for (int j = 0; j < kMedItems; j++) {
-      const int i = tid * kMedItems + j;
-      unsigned k = 0xFFFFFFFFu;  // padding sorts last
-      if (i < n) {
-        k = (unsigned)colIdx[eS + i];
-        if (k >= (unsigned)N) {
-          bad = true;
-          k = 0u;
-        }
+    for (int i = tid; i < n; i += kMedThreads) {
+      unsigned k = (unsigned)colIdx[eS + i];
+      if (k >= (unsigned)N) {
+        bad = true;
+        k = 0u;
       }
-      keys[j] = k;
+      sBuf[0][i] = k;
     }
     if (bad) atomicOr(&hdr->error, 1);
-    // one bit above the column ids keeps the padding behind every real key
-    Sort(u.sort).Sort(keys, 0, colBits + 1 < 32 ? colBits + 1 : 32);
-    __syncthreads();
+    // wave v sorts the keys [cb, ce) of every pass's input into their places of its output
+    const int chunk = ((n + kMedThreads - 1) / kMedThreads) * 64;
+    const int cb = min(n, wave * chunk), ce = min(n, cb + chunk);
+    uint32_t* src = sBuf[0];
+    uint32_t* dst = sBuf[1];
+    uint32_t* hist = sHist[wave];
+    for (int shift = 0; shift < colBits; shift += 8) {
 #pragma unroll
-    for (int j = 0; j < kMedItems; j++) u.keys[tid * kMedItems + j] = keys[j];
+      for (int k = 0; k < 4; k++) hist[lane + 64 * k] = 0;
+      __syncthreads();  // the keys of this pass are in place, the counters are clear
+      for (int i = cb + lane; i < ce; i += 64) atomicAdd(&hist[(src[i] >> shift) & 255u], 1u);
+      __syncthreads();
+      {
+        // thread d: keys with a smaller digit, then this digit's keys of the waves in front
+        unsigned c[WAVES], tot = 0;
+#pragma unroll
+        for (int v = 0; v < WAVES; v++) {
+          c[v] = sHist[v][tid];
+          tot += c[v];
+        }
+        const unsigned incl = wave_inclusive_scan(tot, lane);
+        if (lane == 63) sWaveTot[wave] = incl;
+        __syncthreads();
+        unsigned run = incl - tot;
+#pragma unroll
+        for (int v = 0; v < WAVES; v++)
+          if (v < wave) run += sWaveTot[v];
+#pragma unroll
+        for (int v = 0; v < WAVES; v++) {
+          sHist[v][tid] = run;
+          run += c[v];
+        }
+      }
+      __syncthreads();
+      for (int base = cb; base < ce; base += 64) {
+        const int i = base + lane;
+        const bool valid = i < ce;
+        const uint32_t key = valid ? src[i] : 0u;
+        const unsigned dgt = (key >> shift) & 255u;
+        unsigned long long peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+          const unsigned long long bal = __ballot((dgt >> b) & 1u);
+          peers &= ((dgt >> b) & 1u) ? bal : ~bal;
+        }
+        if (valid) dst[hist[dgt] + __popcll(peers & ltMask)] = key;
+        // the last peer advances the digit's position; the wave's LDS operations stay in order
+        if (valid && (peers >> lane) == 1ull) hist[dgt] += __popcll(peers);
+      }
+      uint32_t* t = src;
+      src = dst;
+      dst = t;
+    }
     __syncthreads();
-    // distinct columns: first occurrences, compacted in order
+    // distinct columns: first occurrences, compacted in order into the other buffer
+    uint32_t* uniq = dst;
+    unsigned keys[kMedItems];
     unsigned cnt = 0;
     unsigned firstMask = 0;
 #pragma unroll
     for (int j = 0; j < kMedItems; j++) {
       const int i = tid * kMedItems + j;
-      const bool first = i < n && (i == 0 || u.keys[i - 1] != keys[j]);
+      keys[j] = i < n ? src[i] : 0u;
+      const bool first = i < n && (i == 0 || src[i - 1] != keys[j]);
       firstMask |= first ? (1u << j) : 0u;
       cnt += first ? 1u : 0u;
     }
@@ -559,7 +605,7 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
     __syncthreads();
     unsigned waveOff = 0, nUniq = 0;
 #pragma unroll
-    for (int v = 0; v < kMedThreads / 64; v++) {
+    for (int v = 0; v < WAVES; v++) {
       const unsigned x = sWaveTot[v];
       if (v < wave) waveOff += x;
       nUniq += x;
@@ -567,7 +613,7 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
     unsigned pos = waveOff + incl - cnt;
 #pragma unroll
     for (int j = 0; j < kMedItems; j++)
-      if ((firstMask >> j) & 1u) sUniq[pos++] = keys[j];
+      if ((firstMask >> j) & 1u) uniq[pos++] = keys[j];
     __syncthreads();
     for (int e = eS + tid; e < eE; e += kMedThreads) {
       unsigned col = (unsigned)colIdx[e];
@@ -575,7 +621,7 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
       int lo = 0, hi = (int)nUniq - 1, found = 0;
       while (lo <= hi) {
         const int mid = (lo + hi) >> 1;
-        const unsigned v = sUniq[mid];
+        const unsigned v = uniq[mid];
         if (v == col) {
           found = mid;
           break;

@@ -63,7 +63,10 @@ __device__ __forceinline__ unsigned cu_key() {
 // leave it behind); launches of this form must not overlap on one device.
 static __device__ int g_windowCursor = 0;
 
-static inline __global__ void reset_window_cursor_kernel() { g_windowCursor = 0; }
+template <int UNUSED = 0>
+__global__ void reset_window_cursor_kernel() {
+  g_windowCursor = 0;
+}
 
 // WIDE: 64-bit row offsets in the K / V gathers.
 template <typename ET, int D, int NWAVES, bool SOFTMAX, bool CLOCKED, bool HEADS, bool W8,
@@ -273,7 +276,7 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
           &perCu, reinterpret_cast<const void*>(kernel), NWAVES * 64, lds));
       unsigned grid = (unsigned)(nCu * (perCu > 0 ? perCu : 1));
       if (grid > gw) grid = gw;
-      hipLaunchKernelGGL(reset_window_cursor_kernel, dim3(1), dim3(1), 0, stream);
+      hipLaunchKernelGGL(reset_window_cursor_kernel<0>, dim3(1), dim3(1), 0, stream);
       hipLaunchKernelGGL(kernel, dim3(grid), block, lds, stream, rwo, order, atox, bm, N, nRW,
                          hl.nTcb, q, k, v, scaleLog2, out, cuTimer, 1, D, D, (float*)nullptr,
                          hl.minBlocks, (int)gw);

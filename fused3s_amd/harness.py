@@ -83,6 +83,50 @@ def tcb_stats(rowPtr, rowWindowOffset, tcblockOffset):
     return out
 
 
+def column_sharing(rowWindowOffset, sparseAToXidx, order, groups=(2, 4, 8), hubs=(2048, 8192)):
+    """How many K / V rows windows that run next to each other have in common, from preprocessing
+    outputs (torch tensors on any device, 16-column blocks). Decides whether gathering a row once
+    for several windows could pay.
+
+    Returns {"pairs": distinct (window, column) pairs,
+             "union_over_sum_<g>": for groups of g windows adjacent in `order` (sortedRowWindows,
+                 or None for natural order): distinct (group, column) pairs / pairs, i.e. the
+                 share of gathered rows that would remain if a group fetched each of its columns
+                 once,
+             "hub_coverage_<h>": share of the pairs that name one of the h most popular columns}.
+    A window's columns are its ascending compacted ids; the slots its last block leaves unused
+    hold 0 and are told apart from column 0 by not ascending."""
+    import torch
+    rwo = rowWindowOffset.to(torch.int64)
+    a = sparseAToXidx.to(torch.int64)
+    nrw = rwo.numel() - 1
+    slots = a.numel()
+    if slots == 0:
+        return {"pairs": 0}
+    win = torch.repeat_interleave(torch.arange(nrw, device=a.device), (rwo[1:] - rwo[:-1]) * 16)
+    first = torch.ones(slots, dtype=torch.bool, device=a.device)
+    first[1:] = win[1:] != win[:-1]
+    valid = first.clone()
+    valid[1:] |= a[1:] > a[:-1]
+    cols, win = a[valid], win[valid]
+    ncol = int(cols.max()) + 1
+    pairs = int(cols.numel())
+    out = {"pairs": pairs}
+    pos = torch.empty(nrw, dtype=torch.int64, device=a.device)
+    if order is None:
+        pos = torch.arange(nrw, device=a.device)
+    else:
+        pos[order.to(torch.int64)] = torch.arange(nrw, device=a.device)
+    for g in groups:
+        grp = torch.div(pos[win], g, rounding_mode="floor")
+        out["union_over_sum_%d" % g] = float(torch.unique(grp * ncol + cols).numel()) / pairs
+    popularity = torch.bincount(cols, minlength=ncol)
+    ranked = torch.sort(popularity, descending=True).values
+    for h in hubs:
+        out["hub_coverage_%d" % h] = float(ranked[:h].sum()) / pairs
+    return out
+
+
 def gpu_model():
     import torch
     if torch.cuda.is_available():
@@ -138,6 +182,9 @@ def run_dataset(name, rowPtr, colIdx, n, algs, embedding_dim=64, n_warp_per_bloc
             runtime[a], throughput[a] = time_kernel(calls[a], flop, niter)
         if stats:
             st = tcb_stats(rowPtr, rwo.cpu().numpy(), toff.cpu().numpy())
+            for tag, od in (("heavy_first_", order), ("natural_", None)):
+                for k, v in column_sharing(rwo, atox, od).items():
+                    st[("" if k == "pairs" else tag) + k] = v
     return runtime, throughput, st
 
 

@@ -47,6 +47,39 @@ def test_tcb_stats_against_direct_counts(oracle_mod):
         harness.tcb_stats(rowPtr, pre["rowWindowOffset"], broken)
 
 
+def test_column_sharing_against_python_sets(oracle_mod):
+    """harness.column_sharing against sets built row by row from the CSR (column 0 present and
+    absent, windows without edges, a last group that is not full)."""
+    import torch
+    from fused3s_amd import harness
+    rng = np.random.default_rng(8)
+    N = 330
+    rowPtr, colIdx = random_csr(rng, N, 12, hub=7, empty_frac=0.25)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    nrw = (N + 15) // 16
+    sets = [set(colIdx[rowPtr[16 * w]:rowPtr[min(16 * w + 16, N)]].tolist()) for w in range(nrw)]
+    assert any(0 in s for s in sets) and any(0 not in s and s for s in sets)
+    pairs = sum(len(s) for s in sets)
+    counts = {}
+    for s in sets:
+        for c in s:
+            counts[c] = counts.get(c, 0) + 1
+    ranked = sorted(counts.values(), reverse=True)
+    for order in (pre["sortedRowWindows"], None):
+        od = None if order is None else torch.as_tensor(order.astype(np.int32))
+        got = harness.column_sharing(torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)),
+                                     torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)), od,
+                                     groups=(2, 4, 8), hubs=(3, 50))
+        assert got["pairs"] == pairs
+        seq = list(range(nrw)) if order is None else [int(w) for w in order]
+        for g in (2, 4, 8):
+            union = sum(len(set().union(*[sets[w] for w in seq[i:i + g]]))
+                        for i in range(0, nrw, g))
+            assert got["union_over_sum_%d" % g] == pytest.approx(union / pairs)
+        assert got["hub_coverage_3"] == pytest.approx(sum(ranked[:3]) / pairs)
+        assert got["hub_coverage_50"] == pytest.approx(sum(ranked[:50]) / pairs)
+
+
 @pytest.mark.gpu
 def test_run_and_tables(tmp_path):
     import pandas as pd
