@@ -61,11 +61,32 @@ constexpr int kFillChunkSmall = 128;  // both, for graphs of short windows (one 
 struct WsHeader {
   long long nTcb;
   int error;
-  int nBig;     // entries in the queue
+  int nBig;     // entries in the queue of the bitset kernel (window_rank_kernel)
   int nextBig;  // next entry to hand out
   int maxCount; // largest per-window block count (multi-workgroup finalize)
-  int nextMed;  // next queue entry to hand out to window_rank_sort_kernel
+  int nMed, nextMed;      // queue of window_rank_sort_kernel, windows of up to kMedMax edges
+  int nLarge, nextLarge;  // the same for its launch over the windows of up to kLargeMax edges
 };
+
+// Where the wave-per-window kernels leave the windows that are too long for them: one queue per
+// kernel that takes such windows, chosen by the window's edge count. big == nullptr: no queues
+// (every long window is found by its own workgroup). medMax == 0: everything goes to `big`.
+struct LongQueues {
+  int32_t* med;
+  int32_t* large;
+  int32_t* big;
+  int medMax, largeMax;
+};
+__device__ __forceinline__ void queue_long_window(const LongQueues& q, WsHeader* hdr, int w,
+                                                  int nEdges) {
+  if (!q.big) return;
+  if (nEdges <= q.medMax)
+    q.med[atomicAdd(&hdr->nMed, 1)] = w;
+  else if (nEdges <= q.largeMax)
+    q.large[atomicAdd(&hdr->nLarge, 1)] = w;
+  else
+    q.big[atomicAdd(&hdr->nBig, 1)] = w;
+}
 constexpr size_t kWsHeaderBytes = 256;
 
 // Inclusive prefix sum over the wave's 64 lanes with data-parallel-primitive moves: shifts within
@@ -148,7 +169,7 @@ template <int W>
 __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int nRW,
     int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
-    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, int32_t* __restrict__ bigList) {
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, LongQueues queues) {
   constexpr int WAVES = kBlock / 64;
   __shared__ uint32_t sKeys[WAVES][kSortMax];
   __shared__ uint32_t sUniq[WAVES][kSortMax];
@@ -168,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_small_kernel(
     return;
   }
   if (n > kSortMax) {  // left to window_rank_kernel, through the queue if there is one
-    if (bigList && lane == 0) bigList[atomicAdd(&hdr->nBig, 1)] = w;
+    if (lane == 0) queue_long_window(queues, hdr, w, n);
     return;
   }
   uint32_t* keys = sKeys[wave];
@@ -274,7 +295,7 @@ template <int W>
 __global__ __launch_bounds__(kBlock) void window_rank_radix_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int nRW,
     int colBits, int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
-    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, int32_t* __restrict__ bigList) {
+    int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr, LongQueues queues) {
   constexpr int WAVES = kBlock / 64;
   constexpr int IDX_BITS = 10;
   static_assert(kSortMax <= (1 << IDX_BITS), "edge position must fit IDX_BITS");
@@ -297,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void window_rank_radix_kernel(
     return;
   }
   if (n > kSortMax) {  // left to window_rank_kernel, through the queue if there is one
-    if (bigList && lane == 0) bigList[atomicAdd(&hdr->nBig, 1)] = w;
+    if (lane == 0) queue_long_window(queues, hdr, w, n);
     return;
   }
   uint32_t* src = sBufA[wave];
@@ -372,7 +393,7 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
     int nPasses, int32_t* __restrict__ blockPartition,
     int32_t* __restrict__ edgeToColumn,
     int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
-    const int32_t* __restrict__ bigList, int skipUpTo) {
+    const int32_t* __restrict__ bigList) {
   extern __shared__ __align__(16) uint32_t smem[];
   uint32_t* bits = smem;                 // range/32 words
   uint32_t* pref = smem + (range >> 5);  // range/128 group prefixes
@@ -400,7 +421,6 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
   __syncthreads();
   const int eS = sRow[0], eE = sRow[16];
   if (!bigList && eE - eS <= kSortMax) break;  // ranked by window_rank_small_kernel
-  if (bigList && eE - eS <= skipUpTo) continue;  // ranked by window_rank_sort_kernel
   const int nGroups = range >> 7;
   unsigned uniqueBefore = 0;
   for (int pass = 0; pass < nPasses; pass++) {
@@ -489,19 +509,30 @@ __global__ __launch_bounds__(TB) void window_rank_kernel(
 // sort of window_rank_radix_kernel widened to a workgroup: eight bits per pass, every wave on its
 // own contiguous quarter of the keys (histogram with LDS atomics, one thread per digit turns the
 // per-wave counts into start positions, in-order scatter with wave ballots), two LDS buffers.
+// Two sizes: windows of up to kMedMax edges (256 threads, 32 KiB of buffers, four workgroups per
+// CU), and the handful of windows of up to kLargeMax edges (1024 threads, 128 KiB), which would
+// otherwise each walk the bitset passes alone at the end of the phase.
 constexpr int kMedThreads = 256;
 constexpr int kMedItems = 16;
 constexpr int kMedMax = kMedThreads * kMedItems;
+constexpr int kLargeThreads = 1024;
+constexpr int kLargeItems = 16;
+constexpr int kLargeMax = kLargeThreads * kLargeItems;
 
-template <int W>
-__global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
+// takes the windows of `queue` (each of at most THREADS * ITEMS edges)
+template <int W, int ITEMS, int THREADS>
+__global__ __launch_bounds__(THREADS) void window_rank_sort_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int colBits,
     int32_t* __restrict__ blockPartition, int32_t* __restrict__ edgeToColumn,
     int32_t* __restrict__ edgeToRow, WsHeader* __restrict__ hdr,
-    const int32_t* __restrict__ bigList) {
-  constexpr int WAVES = kMedThreads / 64;
-  static_assert(kMedThreads == 256, "one thread per 8-bit digit");
-  __shared__ uint32_t sBuf[2][kMedMax];
+    const int32_t* __restrict__ queue, const int* __restrict__ queueLen,
+    int* __restrict__ nextEntry) {
+  constexpr int WAVES = THREADS / 64;
+  constexpr int CAP = THREADS * ITEMS;
+  static_assert(THREADS >= 256 && THREADS % 256 == 0, "the first 256 threads own one digit each");
+  extern __shared__ __align__(16) uint32_t sBufDyn[];  // two buffers of CAP keys
+  uint32_t* const sBuf0 = sBufDyn;
+  uint32_t* const sBuf1 = sBufDyn + CAP;
   __shared__ uint32_t sHist[WAVES][256];
   __shared__ int sRow[17];
   __shared__ unsigned sWaveTot[WAVES];
@@ -510,34 +541,34 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const unsigned long long ltMask = (1ull << lane) - 1ull;
-  const int nBig = hdr->nBig;
+  const int nQueued = *queueLen;
   while (true) {
     __syncthreads();
-    if (tid == 0) sTake = atomicAdd(&hdr->nextMed, 1);
+    if (tid == 0) sTake = atomicAdd(nextEntry, 1);
     __syncthreads();
-    if (sTake >= nBig) break;
-    const int w = bigList[sTake];
+    if (sTake >= nQueued) break;
+    const int w = queue[sTake];
     const int r0 = w * 16;
     if (tid < 17) sRow[tid] = rowPtr[min(r0 + tid, N)];
     __syncthreads();
     const int eS = sRow[0], eE = sRow[16];
     const int n = eE - eS;
-    if (n > kMedMax) continue;  // left to window_rank_kernel
+    if (n > CAP) continue;  // cannot happen: the queue holds what fits
     bool bad = false;
-    for (int i = tid; i < n; i += kMedThreads) {
+    for (int i = tid; i < n; i += THREADS) {
       unsigned k = (unsigned)colIdx[eS + i];
       if (k >= (unsigned)N) {
         bad = true;
         k = 0u;
       }
-      sBuf[0][i] = k;
+      sBuf0[i] = k;
     }
     if (bad) atomicOr(&hdr->error, 1);
     // wave v sorts the keys [cb, ce) of every pass's input into their places of its output
-    const int chunk = ((n + kMedThreads - 1) / kMedThreads) * 64;
+    const int chunk = ((n + THREADS - 1) / THREADS) * 64;
     const int cb = min(n, wave * chunk), ce = min(n, cb + chunk);
-    uint32_t* src = sBuf[0];
-    uint32_t* dst = sBuf[1];
+    uint32_t* src = sBuf0;
+    uint32_t* dst = sBuf1;
     uint32_t* hist = sHist[wave];
     for (int shift = 0; shift < colBits; shift += 8) {
 #pragma unroll
@@ -546,24 +577,28 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
       for (int i = cb + lane; i < ce; i += 64) atomicAdd(&hist[(src[i] >> shift) & 255u], 1u);
       __syncthreads();
       {
-        // thread d: keys with a smaller digit, then this digit's keys of the waves in front
-        unsigned c[WAVES], tot = 0;
+        // thread d < 256: keys with a smaller digit, then this digit's keys of the waves in front
+        unsigned c[WAVES], tot = 0, incl = 0;
+        if (tid < 256) {
 #pragma unroll
-        for (int v = 0; v < WAVES; v++) {
-          c[v] = sHist[v][tid];
-          tot += c[v];
+          for (int v = 0; v < WAVES; v++) {
+            c[v] = sHist[v][tid];
+            tot += c[v];
+          }
+          incl = wave_inclusive_scan(tot, lane);
+          if (lane == 63) sWaveTot[wave] = incl;
         }
-        const unsigned incl = wave_inclusive_scan(tot, lane);
-        if (lane == 63) sWaveTot[wave] = incl;
         __syncthreads();
-        unsigned run = incl - tot;
+        if (tid < 256) {
+          unsigned run = incl - tot;
 #pragma unroll
-        for (int v = 0; v < WAVES; v++)
-          if (v < wave) run += sWaveTot[v];
+          for (int v = 0; v < 4; v++)
+            if (v < wave) run += sWaveTot[v];
 #pragma unroll
-        for (int v = 0; v < WAVES; v++) {
-          sHist[v][tid] = run;
-          run += c[v];
+          for (int v = 0; v < WAVES; v++) {
+            sHist[v][tid] = run;
+            run += c[v];
+          }
         }
       }
       __syncthreads();
@@ -587,35 +622,33 @@ __global__ __launch_bounds__(kMedThreads) void window_rank_sort_kernel(
       dst = t;
     }
     __syncthreads();
-    // distinct columns: first occurrences, compacted in order into the other buffer
+    // distinct columns: first occurrences, compacted in order into the other buffer (every wave
+    // on its quarter [cb, ce) again: a count with ballots, the waves' totals, then the stores)
     uint32_t* uniq = dst;
-    unsigned keys[kMedItems];
     unsigned cnt = 0;
-    unsigned firstMask = 0;
-#pragma unroll
-    for (int j = 0; j < kMedItems; j++) {
-      const int i = tid * kMedItems + j;
-      keys[j] = i < n ? src[i] : 0u;
-      const bool first = i < n && (i == 0 || src[i - 1] != keys[j]);
-      firstMask |= first ? (1u << j) : 0u;
-      cnt += first ? 1u : 0u;
+    for (int base = cb; base < ce; base += 64) {
+      const int i = base + lane;
+      const bool first = i < ce && (i == 0 || src[i - 1] != src[i]);
+      cnt += (unsigned)__popcll(__ballot(first));
     }
-    const unsigned incl = wave_inclusive_scan(cnt, lane);
-    if (lane == 63) sWaveTot[wave] = incl;
+    if (lane == 0) sWaveTot[wave] = cnt;
     __syncthreads();
-    unsigned waveOff = 0, nUniq = 0;
+    unsigned pos = 0, nUniq = 0;
 #pragma unroll
     for (int v = 0; v < WAVES; v++) {
       const unsigned x = sWaveTot[v];
-      if (v < wave) waveOff += x;
+      if (v < wave) pos += x;
       nUniq += x;
     }
-    unsigned pos = waveOff + incl - cnt;
-#pragma unroll
-    for (int j = 0; j < kMedItems; j++)
-      if ((firstMask >> j) & 1u) uniq[pos++] = keys[j];
+    for (int base = cb; base < ce; base += 64) {
+      const int i = base + lane;
+      const bool first = i < ce && (i == 0 || src[i - 1] != src[i]);
+      const unsigned long long bal = __ballot(first);
+      if (first) uniq[pos + (unsigned)__popcll(bal & ltMask)] = src[i];
+      pos += (unsigned)__popcll(bal);
+    }
     __syncthreads();
-    for (int e = eS + tid; e < eE; e += kMedThreads) {
+    for (int e = eS + tid; e < eE; e += THREADS) {
       unsigned col = (unsigned)colIdx[e];
       if (col >= (unsigned)N) col = 0u;
       int lo = 0, hi = (int)nUniq - 1, found = 0;
@@ -1182,9 +1215,9 @@ __device__ __forceinline__ void fill_window_generic(
 // leave LDS as contiguous runs. A window with a repeated or descending column is handed to
 // fill_window_generic. TC blocks of LDS at a time on the short way, TCG on the general one.
 template <int W, int TB, int TC, int TCG>
-__global__ __launch_bounds__(TB) void window_fill_kernel(
-    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
-    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
+__device__ __forceinline__ void fill_one_window(
+    int w, int nRW, const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N,
+    int E, const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
     const WsHeader* __restrict__ hdr, int32_t* __restrict__ tcblockRowid,
     uint8_t* __restrict__ tcblocktileId, int32_t* __restrict__ tcblockOffset,
     int32_t* __restrict__ sparseAToXidx, unsigned long long* __restrict__ bitmap, int minBlocks,
@@ -1204,12 +1237,11 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int w = blockIdx.x;
   // launched right behind phase 1 (no host in between): a column index outside [0, N) left
   // edgeToColumn unwritten, so nothing here may run
   if (hdr && hdr->error) return;
   if (tid == 0) sUnsorted = 0u;
-  if (w == 0 && tid == 0) tcblockOffset[rowWindowOffset[gridDim.x]] = E;
+  if (w == 0 && tid == 0) tcblockOffset[rowWindowOffset[nRW]] = E;
   const int base = rowWindowOffset[w];
   const int nb = rowWindowOffset[w + 1] - base;
   // a launch may be one of two that share the windows by length: [minBlocks, maxBlocks]
@@ -1333,6 +1365,52 @@ __global__ __launch_bounds__(TB) void window_fill_kernel(
     fill_window_generic<W, TB>(colIdx, edgeToColumn, w, base, nb, TCG, tcblockRowid,
                                tcblocktileId, tcblockOffset, sparseAToXidx, bitmap, gCnt, gBm, sRow,
                                sWaveTot, &sUnsorted);
+  }
+}
+
+template <int W, int TB, int TC, int TCG>
+__global__ __launch_bounds__(TB) void window_fill_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
+    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
+    const WsHeader* __restrict__ hdr, int32_t* __restrict__ tcblockRowid,
+    uint8_t* __restrict__ tcblocktileId, int32_t* __restrict__ tcblockOffset,
+    int32_t* __restrict__ sparseAToXidx, unsigned long long* __restrict__ bitmap, int minBlocks,
+    int maxBlocks) {
+  fill_one_window<W, TB, TC, TCG>((int)blockIdx.x, (int)gridDim.x, rowPtr, colIdx, N, E,
+                                  edgeToColumn, rowWindowOffset, hdr, tcblockRowid, tcblocktileId,
+                                  tcblockOffset, sparseAToXidx, bitmap, minBlocks, maxBlocks);
+}
+
+// The few long windows of a graph of short ones (more than minBlocks - 1 TC blocks): a grid of a
+// few hundred workgroups looks through the block counts, 256 windows at a time per workgroup,
+// and fills the long ones it finds one after the other. One workgroup per window, as
+// window_fill_kernel has it, would start a hundred thousand workgroups of 60 KiB of LDS each to
+// find that nearly all of them have nothing to do.
+template <int W, int TB, int TC, int TCG>
+__global__ __launch_bounds__(TB) void window_fill_long_kernel(
+    const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E, int nRW,
+    const int32_t* __restrict__ edgeToColumn, const int32_t* __restrict__ rowWindowOffset,
+    const WsHeader* __restrict__ hdr, int32_t* __restrict__ tcblockRowid,
+    uint8_t* __restrict__ tcblocktileId, int32_t* __restrict__ tcblockOffset,
+    int32_t* __restrict__ sparseAToXidx, unsigned long long* __restrict__ bitmap, int minBlocks) {
+  static_assert(TB == 256, "one candidate window per thread and round");
+  __shared__ int sList[TB];
+  __shared__ int sListLen;
+  for (int base = (int)blockIdx.x * TB; base < nRW; base += (int)gridDim.x * TB) {
+    __syncthreads();  // the previous round's list has been worked through
+    if (threadIdx.x == 0) sListLen = 0;
+    __syncthreads();
+    const int w = base + (int)threadIdx.x;
+    if (w < nRW && rowWindowOffset[w + 1] - rowWindowOffset[w] >= minBlocks)
+      sList[atomicAdd(&sListLen, 1)] = w;
+    __syncthreads();
+    const int len = sListLen;
+    for (int k = 0; k < len; k++) {
+      __syncthreads();  // the window before this one has left the LDS arrays
+      fill_one_window<W, TB, TC, TCG>(sList[k], nRW, rowPtr, colIdx, N, E, edgeToColumn,
+                                      rowWindowOffset, hdr, tcblockRowid, tcblocktileId,
+                                      tcblockOffset, sparseAToXidx, bitmap, minBlocks, 0x7FFFFFFF);
+    }
   }
 }
 
@@ -1758,7 +1836,10 @@ __global__ void clear_header_kernel(WsHeader* hdr) {
   hdr->nBig = 0;
   hdr->nextBig = 0;
   hdr->maxCount = 0;
+  hdr->nMed = 0;
   hdr->nextMed = 0;
+  hdr->nLarge = 0;
+  hdr->nextLarge = 0;
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -1832,6 +1913,9 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
   const int nRW = (N + kWinRows - 1) / kWinRows;
   WsHeader* hdr = reinterpret_cast<WsHeader*>(ws);
   const size_t seg = align256((size_t)nRW * sizeof(int32_t));
+  // the three buffers the window order later sorts in hold the queues of long windows until then
+  int32_t* keysA = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes);
+  int32_t* keysB = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + seg);
   int32_t* valsTmp = reinterpret_cast<int32_t*>(ws + kWsHeaderBytes + 2 * seg);
 
   hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(1), 0, stream, hdr);
@@ -1843,6 +1927,12 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
     const int smallGrid = (nRW + kBlock / 64 - 1) / (kBlock / 64);
     const bool big = (int64_t)E >= (int64_t)nRW * 2048;  // long windows on average
     int32_t* queue = big ? nullptr : valsTmp;
+    // queued windows of a few thousand edges on a graph that needs several bitset passes are
+    // sorted (window_rank_sort_kernel) instead of walking every pass; the others go to the
+    // bitset kernel
+    const bool sortMedium = queue != nullptr && nPasses >= 2;
+    const LongQueues queues = {keysA, keysB, queue, sortMedium ? kMedMax : 0,
+                               sortMedium ? kLargeMax : 0};
     // short windows: radix sort of packed (column, position) words when the column ids leave
     // room for the position, else the bitonic network on bare column ids
     int colBits = 0;
@@ -1851,42 +1941,51 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
       if (W == 16)
         hipLaunchKernelGGL(window_rank_radix_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
                            rowPtr, colIdx, N, nRW, colBits, blockPartition, edgeToColumn,
-                           edgeToRow, hdr, queue);
+                           edgeToRow, hdr, queues);
       else
         hipLaunchKernelGGL(window_rank_radix_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
                            rowPtr, colIdx, N, nRW, colBits, blockPartition, edgeToColumn,
-                           edgeToRow, hdr, queue);
+                           edgeToRow, hdr, queues);
     } else if (W == 16) {
       hipLaunchKernelGGL(window_rank_small_kernel<16>, dim3(smallGrid), dim3(kBlock), 0, stream,
                          rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
-                         queue);
+                         queues);
     } else {
       hipLaunchKernelGGL(window_rank_small_kernel<8>, dim3(smallGrid), dim3(kBlock), 0, stream,
                          rowPtr, colIdx, N, nRW, blockPartition, edgeToColumn, edgeToRow, hdr,
-                         queue);
+                         queues);
     }
     F3S_HIP_CHECK(hipGetLastError());
-    // eight waves per window when windows are long (more loads and LDS atomics in flight)
-    // queued windows of a few thousand edges on a graph that needs several bitset passes are
-    // sorted instead (window_rank_sort_kernel); the bitset kernel then skips them
-    const bool sortMedium = queue != nullptr && nPasses >= 2;
-    const int skipUpTo = sortMedium ? kMedMax : 0;
     if (sortMedium) {
+      // two launches: up to kMedMax edges with 32 KiB of sort buffers (four workgroups per CU),
+      // then the few windows up to kLargeMax with 128 KiB (one per CU)
+#define F3S_SORT(WW, ITEMS, THREADS, GRID, QUEUE, LEN, COUNTER)                                 \
+  do {                                                                                          \
+    constexpr size_t ldsSort = (size_t)2 * THREADS * ITEMS * sizeof(uint32_t);                  \
+    if (ldsSort > 48 * 1024)                                                                    \
+      F3S_HIP_CHECK(hipFuncSetAttribute(                                                        \
+          reinterpret_cast<const void*>(&window_rank_sort_kernel<WW, ITEMS, THREADS>),          \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsSort));                           \
+    hipLaunchKernelGGL((window_rank_sort_kernel<WW, ITEMS, THREADS>), dim3(GRID), dim3(THREADS),\
+                       ldsSort, stream, rowPtr, colIdx, N, colBits, blockPartition,             \
+                       edgeToColumn, edgeToRow, hdr, QUEUE, LEN, COUNTER);                      \
+    F3S_HIP_CHECK(hipGetLastError());                                                           \
+  } while (0)
       const int medGrid = nRW < 1024 ? nRW : 1024;
-      if (W == 16)
-        hipLaunchKernelGGL(window_rank_sort_kernel<16>, dim3(medGrid), dim3(kMedThreads), 0,
-                           stream, rowPtr, colIdx, N, colBits, blockPartition, edgeToColumn,
-                           edgeToRow, hdr, queue);
-      else
-        hipLaunchKernelGGL(window_rank_sort_kernel<8>, dim3(medGrid), dim3(kMedThreads), 0, stream,
-                           rowPtr, colIdx, N, colBits, blockPartition, edgeToColumn, edgeToRow,
-                           hdr, queue);
-      F3S_HIP_CHECK(hipGetLastError());
+      const int largeGrid = nRW < 256 ? nRW : 256;
+      if (W == 16) {
+        F3S_SORT(16, kMedItems, kMedThreads, medGrid, keysA, &hdr->nMed, &hdr->nextMed);
+        F3S_SORT(16, kLargeItems, kLargeThreads, largeGrid, keysB, &hdr->nLarge, &hdr->nextLarge);
+      } else {
+        F3S_SORT(8, kMedItems, kMedThreads, medGrid, keysA, &hdr->nMed, &hdr->nextMed);
+        F3S_SORT(8, kLargeItems, kLargeThreads, largeGrid, keysB, &hdr->nLarge, &hdr->nextLarge);
+      }
+#undef F3S_SORT
     }
 #define F3S_RANK(WW, TBB)                                                                     \
   hipLaunchKernelGGL((window_rank_kernel<WW, TBB>), dim3(rankGrid), dim3(TBB), lds, stream,   \
                      rowPtr, colIdx, N, range, nPasses, blockPartition,                       \
-                     edgeToColumn, edgeToRow, hdr, queue, skipUpTo)
+                     edgeToColumn, edgeToRow, hdr, queue)
     // the queue lives in the buffer finalize_count_kernel later uses for its values and is
     // drained by at most 8 workgroups per CU
     const int rankGrid = big ? nRW : (nRW < 2048 ? nRW : 2048);
@@ -2010,6 +2109,12 @@ int enqueue_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int
   hipLaunchKernelGGL((window_fill_kernel<WW, TBB, TCC, TCG>), dim3(nRW), dim3(TBB), 0, stream, \
                      rowPtr, colIdx, N, E, edgeToColumn, rowWindowOffset, hdr, tcblockRowid,   \
                      tcblocktileId, tcblockOffset, sparseAToXidx, bm, LO, HI)
+  // the long windows of a graph of short ones: at most two workgroups per CU look for them
+#define F3S_FILL_LONG(WW)                                                                       \
+  hipLaunchKernelGGL((window_fill_long_kernel<WW, 256, kFillChunk, kFillChunkGeneric>),         \
+                     dim3((unsigned)min(512, (nRW + 255) / 256)), dim3(256), 0, stream, rowPtr, \
+                     colIdx, N, E, nRW, edgeToColumn, rowWindowOffset, hdr, tcblockRowid,       \
+                     tcblocktileId, tcblockOffset, sparseAToXidx, bm, kFillChunkSmall + 1)
   const bool big = (int64_t)E >= (int64_t)nRW * 2048;
   constexpr int kAll = 0x7FFFFFFF;
   if (W == 16) {
@@ -2018,7 +2123,7 @@ int enqueue_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int
     } else {
       F3S_FILL(16, 64, kFillChunkSmall, kFillChunkSmall, 0, kFillChunkSmall);
       F3S_HIP_CHECK(hipGetLastError());
-      F3S_FILL(16, 256, kFillChunk, kFillChunkGeneric, kFillChunkSmall + 1, kAll);
+      F3S_FILL_LONG(16);
     }
   } else {
     if (big) {
@@ -2026,10 +2131,11 @@ int enqueue_fill(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int
     } else {
       F3S_FILL(8, 64, kFillChunkSmall, kFillChunkSmall, 0, kFillChunkSmall);
       F3S_HIP_CHECK(hipGetLastError());
-      F3S_FILL(8, 256, kFillChunk, kFillChunkGeneric, kFillChunkSmall + 1, kAll);
+      F3S_FILL_LONG(8);
     }
   }
 #undef F3S_FILL
+#undef F3S_FILL_LONG
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
 }
