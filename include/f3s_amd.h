@@ -77,7 +77,9 @@ int f3s_preprocess_count(const int32_t* rowPtr, const int32_t* colIdx, int N, in
  * enqueued on `stream` (kernels only, no memset nodes). Every call on a GPU shares that GPU's
  * buffer: calls that overlap on one GPU (different streams, different threads) race; calls that
  * follow each other on one stream, or are otherwise ordered, are safe, and each call clears what
- * it needs cleared.
+ * it needs cleared. The first call on a device looks up the buffer's address
+ * (hipGetSymbolAddress) and may set a kernel attribute (hipFuncSetAttribute): make that call
+ * outside stream capture; the calls after it only launch kernels.
  */
 size_t f3s_preprocess_static_scratch_bytes(void);
 int f3s_preprocess_count_static(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, int H,

@@ -259,3 +259,42 @@ def test_rows_beyond_4_gib(oracle_mod):
         del os.environ["F3S_SCHEDULE"]
     assert np.abs(got - want).max() < MAX_ABS
     assert mean_rel(got, want) < MEAN_REL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sliced", [True, False])
+def test_attention_call_under_graph_capture(oracle_mod, long_window_graph, sliced):
+    """f3s_attention_fwd only launches kernels (no host wait, no copy, no allocation), so a call
+    can be captured into a HIP graph, the very first call on a workspace included. Three replays
+    with eager work and synchronisations between them, each against the eager result; new Q
+    values written into the captured input buffer between replays show up in the output."""
+    from fused3s_amd import capi
+    print("case graph capture sliced=%s" % sliced, flush=True)
+    N, _, _, pre = long_window_graph
+    d = 64
+    rng = np.random.default_rng(13)
+    Q, K, V = [torch.as_tensor(rng.standard_normal((N, d)).astype(np.float16)).cuda()
+               for _ in range(3)]
+    rwo, order, atox, bm = to_dev(pre)
+    ws = capi.attention_workspace(N, d, "cuda", nTCB=int(pre["blockCount"])) if sliced else None
+    out = torch.empty((N, d), dtype=torch.float32, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            capi.attention(rwo, order, atox, bm, N, Q, K, V, 8.0, out=out, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        if rep:
+            Q.copy_(torch.as_tensor(rng.standard_normal((N, d)).astype(np.float16)))
+        out.fill_(-3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = capi.attention(rwo, order, atox, bm, N, Q, K, V, 8.0, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), "replay %d" % rep
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                    pre["tcbBitMap"], N, bits(Q), bits(K), bits(V), 8.0)
+    assert np.abs(got.cpu().numpy() - want).max() < MAX_ABS

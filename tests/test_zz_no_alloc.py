@@ -41,8 +41,16 @@ def test_static_scratch_matches_workspace_entry_twice(W):
         rp, ci = _graph(seed, N, deg, **kw)
         want = capi.preprocess(rp, ci, N, 16, W)
         got = _buffers(N, int(ci.numel()), -7)
+        torch.cuda.synchronize()
+        # the property the entry exists for: with the caller's buffers in place, the call takes
+        # no device memory (neither through torch nor beside it); the very first call on a device
+        # looks up the scratch array's address, which allocates nothing either
+        free_before, _ = torch.cuda.mem_get_info()
+        torch_before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
         capi.preprocess_count_static(rp, ci, N, got, 16, W)
         torch.cuda.synchronize()
+        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == torch_before
+        assert torch.cuda.mem_get_info()[0] == free_before
         for k in KEYS:
             assert torch.equal(got[k], want[k]), k
         assert got["result"].tolist() == [want["blockCount"], 0]
