@@ -118,6 +118,24 @@ def cpu_baseline_torch(rowPtr, colIdx, N, Q, K, V, scale, d, max_edges=4_000_000
                       "%d rows (%d edges), %.2f s" % (rows_n, e, dt)}
 
 
+def bucketed_order(pre, N, buckets):
+    """An experimental launch order (results do not depend on the order): windows grouped by the
+    column range (one of `buckets` equal parts) that most of their TC blocks start in, heavy
+    windows first inside a group. For graphs whose K + V exceed the caches, so that windows that
+    run together name neighbouring rows."""
+    import torch
+    rwo = pre["rowWindowOffset"].long()
+    nrw = rwo.numel() - 1
+    counts = rwo[1:] - rwo[:-1]
+    first_col = pre["sparseAToXidx"].view(-1, 16)[:, 0].long()
+    win = torch.repeat_interleave(torch.arange(nrw, device=rwo.device), counts)
+    part = torch.clamp(first_col * buckets // max(N, 1), max=buckets - 1)
+    hist = torch.bincount(win * buckets + part, minlength=nrw * buckets).view(nrw, buckets)
+    bucket = hist.argmax(dim=1)
+    key = bucket * (int(counts.max()) + 1) + (int(counts.max()) - counts)
+    return torch.argsort(key, stable=True).to(torch.int32)
+
+
 def recorded_traffic(config, schedule, scale, natural_order):
     """HBM-side bytes per attention call as rocprofv3 counted them in an EARLIER run (FETCH_SIZE
     and WRITE_SIZE, scaled by what the same counters read for a plain copy): counters cannot be
@@ -189,6 +207,8 @@ def run_config(name, args, dev, headline):
 
     natural = headline and args.natural_order
     order = None if natural else pre["sortedRowWindows"]
+    if headline and args.column_buckets > 0:
+        order = bucketed_order(pre, N, args.column_buckets)
     out = torch.empty((N, heads * d), dtype=torch.float32, device=dev)
     # scratch of the column-sliced schedule, which the library picks for graphs with long windows
     workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype,
@@ -283,7 +303,9 @@ def run_config(name, args, dev, headline):
                                % (name, N, E, d, cfg["dtype"],
                                   "single head" if heads == 1 else
                                   "%d heads in one launch, output [N, %d]" % (heads, D),
-                                  "natural" if natural else "heavy-first"),
+                                  "natural" if natural else
+                                  "%d column groups, heavy-first inside" % args.column_buckets
+                                  if headline and args.column_buckets > 0 else "heavy-first"),
                    "nTCB": nTCB, "nRW": nRW, "max_tcb_per_window": int(cnt.max()),
                    "max_degree": max_degree, "scale": scale_graph},
         "kernel_ms_median": t_med * 1e3, "kernel_ms_mean": t_avg * 1e3,
@@ -343,6 +365,9 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the compact lines of the other benchmark configurations")
     ap.add_argument("--natural-order", action="store_true", help="launch windows in natural order")
+    ap.add_argument("--column-buckets", type=int, default=0,
+                    help="experiment: launch windows grouped by the column range most of their "
+                         "blocks start in (this many ranges), heavy-first inside a group")
     ap.add_argument("--two-phase-preprocess", action="store_true",
                     help="preprocess with f3s_preprocess_count + f3s_preprocess_fill instead of "
                          "the one call f3s_preprocess")

@@ -202,6 +202,10 @@ CONFIGS = {
     # with (p_in = 0.02 gives ~0.6 M)
     "cfg5b_sbm_100k_dense": dict(kind="sbm", N=100000, n_blocks=500, p_in=0.2, p_out=1e-5, d=32,
                                  dtype="bf16", heads=8),
+    # not one of the benchmark's configurations: the multi-head layer of configuration 5 on the
+    # long-window graph of configuration 3 (the multi-head entry with the column-sliced schedule)
+    "extra_chunglu_233k_8x32": dict(kind="chunglu", N=232965, E=114_600_000, gamma=2.1,
+                                    max_degree=26000, d=32, dtype="bf16", heads=8),
 }
 
 
