@@ -1987,8 +1987,8 @@ int enqueue_count(const int32_t* rowPtr, const int32_t* colIdx, int N, int E, in
                      rowPtr, colIdx, N, range, nPasses, blockPartition,                       \
                      edgeToColumn, edgeToRow, hdr, queue)
     // the queue lives in the buffer finalize_count_kernel later uses for its values and is
-    // drained by at most 8 workgroups per CU
-    const int rankGrid = big ? nRW : (nRW < 2048 ? nRW : 2048);
+    // drained by at most two workgroups per CU (2048 of them took 25 us to find an empty queue)
+    const int rankGrid = big ? nRW : (nRW < 512 ? nRW : 512);
     if (W == 16) {
       if (big) F3S_RANK(16, 512); else F3S_RANK(16, 256);
     } else {
