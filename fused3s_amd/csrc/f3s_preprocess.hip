@@ -1397,7 +1397,7 @@ __global__ __launch_bounds__(TB) void window_fill_long_kernel(
   __shared__ int sList[TB];
   __shared__ int sListLen;
   for (int base = (int)blockIdx.x * TB; base < nRW; base += (int)gridDim.x * TB) {
-    __syncthreads();  // the previous round's list has been worked through
+    __syncthreads();  // the list of the 256 windows before these has been worked through
     if (threadIdx.x == 0) sListLen = 0;
     __syncthreads();
     const int w = base + (int)threadIdx.x;
