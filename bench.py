@@ -197,6 +197,16 @@ def run_config(name, args, dev, headline):
         "of the HBM scan bound)" % (nTCB, nRW, int(cnt.max()), float(cnt.float().mean()), pre_ms,
                                     E / pre_ms / 1e6, 100 * pre_hbm_frac))
 
+    if headline and args.preprocess_only:
+        return {"metric": "preprocess_ms", "value": pre_ms, "unit": "ms", "n_gpus": 1,
+                "higher_is_better": False, "data": "synthetic",
+                "config": {"workload": "%s: N=%d E=%d, CSR -> TC blocks" % (name, N, E),
+                           "nTCB": nTCB, "nRW": nRW},
+                "preprocess_gedges_per_s": E / pre_ms / 1e6, "preprocess_hbm_frac": pre_hbm_frac}
+    if os.path.basename(capi.LIB_PATH).startswith("libf3s_amd_pre_"):
+        raise SystemExit("bench.py: %s is a preprocessing probe whose block arrays are incomplete; "
+                         "it may only be timed with --preprocess-only" % capi.LIB_PATH)
+
     if headline and args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)  # 1 GiB
         dst = torch.empty_like(src)
@@ -371,6 +381,8 @@ def main():
     ap.add_argument("--two-phase-preprocess", action="store_true",
                     help="preprocess with f3s_preprocess_count + f3s_preprocess_fill instead of "
                          "the one call f3s_preprocess")
+    ap.add_argument("--preprocess-only", action="store_true",
+                    help="time the preprocessing of --config and stop (no attention call)")
     ap.add_argument("--cpu-budget", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known bytes, for scaling rocprof's "
@@ -388,7 +400,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     result = run_config(args.config, args, dev, headline=True)
-    if not args.no_other_configs:
+    if not args.no_other_configs and not args.preprocess_only:
         # the other benchmark configurations, one compact entry each (kernel time, the bound that
         # binds on paper and the fraction reached, preprocessing time)
         others = []

@@ -46,6 +46,17 @@ PROBES = {
     "no_compute": ["-DF3S_PROBE_NO_COMPUTE"],
     # LDS reads and arithmetic on whatever the first two steps left in the ring, no gather
     "no_gather": ["-DF3S_PROBE_NO_GATHER"],
+    # Preprocessing (window_rank_fill_kernel) with one part left out. Their block arrays are
+    # incomplete: time them with `python bench.py --preprocess-only` and never hand what they
+    # produce to an attention call (bench.py refuses to).
+    # the compacted column ids are not enumerated from the bitset
+    "pre_no_ids": ["-DF3S_PROBE_PRE_NO_IDS"],
+    # no second pass over the window's edges: no ranks, rows, bitmap bits (and so no tile ids)
+    "pre_no_fill": ["-DF3S_PROBE_PRE_NO_FILL"],
+    # the second pass without its edgeToColumn / edgeToRow stores
+    "pre_no_edge_stores": ["-DF3S_PROBE_PRE_NO_EDGE_STORES"],
+    # the tile ids are not walked out of the bitmaps
+    "pre_no_tile_ids": ["-DF3S_PROBE_PRE_NO_TILEIDS"],
 }
 
 

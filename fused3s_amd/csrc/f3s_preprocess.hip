@@ -703,12 +703,32 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   const int cBegin = min(wave * chunk, nRW);
   const int cEnd = min(cBegin + chunk, nRW);
 
+  // ---- the counts into LDS first, every thread's loads in flight together: each later pass
+  // walks its chunk group by group, and a global load per group would cost its full latency
+  // every time
+  {
+    constexpr int U = 4;
+    for (int i0 = tid; i0 < nRW; i0 += U * kFinBlock) {
+      int v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int i = i0 + u * kFinBlock;
+        v[u] = i < nRW ? blockPartition[i] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int i = i0 + u * kFinBlock;
+        if (i < nRW) bufB[i] = (uint32_t)v[u];
+      }
+    }
+  }
+  __syncthreads();
   // ---- inclusive scan of the block counts into rowWindowOffset[1..], and their maximum
   {
     unsigned sum = 0;
     int mx = 0;
     for (int i = cBegin + lane; i < cEnd; i += 64) {
-      const int v = blockPartition[i];
+      const int v = (int)bufB[i];
       sum += (unsigned)v;
       mx = max(mx, v);
     }
@@ -734,7 +754,7 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
   }
   for (int base = cBegin; base < cEnd; base += 64) {
     const int i = base + lane;
-    const unsigned v = (i < cEnd) ? (unsigned)blockPartition[i] : 0u;
+    const unsigned v = (i < cEnd) ? bufB[i] : 0u;
     const unsigned incl = wave_inclusive_scan(v, lane);
     if (i < cEnd) rowWindowOffset[i + 1] = (int)(carry + incl);
     carry += __shfl(incl, 63);
@@ -773,20 +793,14 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     };
     auto load_key = [&](int i) -> unsigned {
       if (i >= cEnd) return 0u;
-      return pass == 0 ? ((unsigned)(maxC - blockPartition[i]) << kFinIdBits) | (unsigned)i
-                       : src[i];
+      // the first pass finds the counts themselves in bufB
+      return pass == 0 ? ((unsigned)(maxC - (int)src[i]) << kFinIdBits) | (unsigned)i : src[i];
     };
-    // histogram of the wave's chunk (the next group's keys are in flight during this one's)
-    unsigned keyNext = load_key(cBegin + lane);
-    for (int base = cBegin; base < cEnd; base += 64) {
-      const int i = base + lane;
-      const bool valid = i < cEnd;
-      const unsigned key = keyNext;
-      keyNext = load_key(i + 64);
-      const int dgt = (int)(key >> shift) & (NB - 1);
-      const unsigned long long peers = digit_peers(valid, dgt);
-      if (valid && (peers & ltMask) == 0ull) sCnt[wave][dgt] += __popcll(peers);
-    }
+    // histogram of the wave's chunk: LDS atomics (the whole workgroup shares one CU's vector
+    // ALUs, and a ballot per digit bit costs far more instructions than the atomic's conflicts)
+    wave_lds_sync();
+    for (int i = cBegin + lane; i < cEnd; i += 64)
+      atomicAdd(&sCnt[wave][(int)(load_key(i) >> shift) & (NB - 1)], 1u);
     __syncthreads();
     // start of (digit = lane, wave): all smaller digits, then the same digit in earlier waves
     unsigned digitTotal = 0, before = 0;
@@ -799,8 +813,8 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     const unsigned start = wave_inclusive_scan(digitTotal, lane) - digitTotal + before;
     __syncthreads();
     sCnt[wave][lane] = start;
-    // scatter, in order
-    keyNext = load_key(cBegin + lane);
+    // scatter, in order (the next group's key is in flight during this one's)
+    unsigned keyNext = load_key(cBegin + lane);
     for (int base = cBegin; base < cEnd; base += 64) {
       const int i = base + lane;
       const bool valid = i < cEnd;
@@ -808,15 +822,16 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
       keyNext = load_key(i + 64);
       const int dgt = (int)(key >> shift) & (NB - 1);
       const unsigned long long peers = digit_peers(valid, dgt);
-      if (valid) {
-        const unsigned pos = sCnt[wave][dgt] + __popcll(peers & ltMask);
-        if (last)
-          sortedRowWindows[pos] = (int)(key & ((1u << kFinIdBits) - 1u));
-        else
-          dst[pos] = key;
-      }
+      if (valid) dst[sCnt[wave][dgt] + __popcll(peers & ltMask)] = key;
       // the last peer moves the digit's running position (the wave's LDS accesses stay in order)
       if (valid && (peers >> lane) == 1ull) sCnt[wave][dgt] += __popcll(peers);
+    }
+    if (last) {
+      // the order leaves LDS as whole lines: scattered 4-byte stores from the last pass would
+      // all go through this one CU's address unit, 64 lines per instruction
+      __syncthreads();
+      for (int i = tid; i < nRW; i += kFinBlock)
+        sortedRowWindows[i] = (int)(dst[i] & ((1u << kFinIdBits) - 1u));
     }
   }
 }
@@ -1548,7 +1563,8 @@ __global__ __launch_bounds__(TB) __attribute__((amdgpu_waves_per_eu(6, 6)))
 void window_rank_fill_kernel(
     const int32_t* __restrict__ rowPtr, const int32_t* __restrict__ colIdx, int N, int E,
     int range, int chunkBytes, const int32_t* __restrict__ rowWindowOffset,
-    const WsHeader* __restrict__ hdr, int32_t* edgeToColumn, int32_t* __restrict__ edgeToRow,
+    const int32_t* __restrict__ order, const WsHeader* __restrict__ hdr, int32_t* edgeToColumn,
+    int32_t* __restrict__ edgeToRow,
     int32_t* __restrict__ tcblockRowid, uint8_t* __restrict__ tcblocktileId,
     int32_t* __restrict__ tcblockOffset, int32_t* __restrict__ sparseAToXidx,
     unsigned long long* __restrict__ bitmap) {
@@ -1573,7 +1589,9 @@ void window_rank_fill_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int w = blockIdx.x;
+  // windows start in the heavy-first order that the scan kernel has just written: the longest
+  // ones first, so that none of them is still running alone when the others are done
+  const int w = order[blockIdx.x];
   if (hdr->error) return;  // a column index outside [0, N): the caller gets the error, no output
   if (w == 0 && tid == 0) tcblockOffset[rowWindowOffset[gridDim.x]] = E;
   const int base = rowWindowOffset[w];
@@ -1628,6 +1646,9 @@ void window_rank_fill_kernel(
       if (i < nW64) {
         unsigned pos = sTot[k * NWAVE + wave] + pref[i];
         pref[i] = pos;
+#ifdef F3S_PROBE_PRE_NO_IDS
+        continue;
+#endif
         // 32 bits at a time, with a 32-bit byte offset from the window's first id slot
         const unsigned long long x = bits64[i];
         unsigned off = pos * 4u;
@@ -1694,8 +1715,10 @@ void window_rank_fill_kernel(
 #pragma unroll
       for (int u = 0; u < 4; u++) ecs[u] = rank_of(cols[u]);
       if (first) {
+#ifndef F3S_PROBE_PRE_NO_EDGE_STORES
         *reinterpret_cast<int4*>(edgeToColumn + e0) = make_int4(ecs[0], ecs[1], ecs[2], ecs[3]);
         *reinterpret_cast<int4*>(edgeToRow + e0) = make_int4(r0 + r, r0 + r, r0 + r, r0 + r);
+#endif
         const bool bad = (e0 > sRow[r] && left >= cols[0]) || cols[0] >= cols[1] ||
                          cols[1] >= cols[2] || cols[2] >= cols[3];
         if (bad) atomicOr(&sUnsorted, 1u << r);
@@ -1729,6 +1752,9 @@ void window_rank_fill_kernel(
         if (m[u]) atomicOr(&sBmWords[word[u]], m[u]);
     };
     // two groups per thread and step, loads first
+#ifdef F3S_PROBE_PRE_NO_FILL
+    if (nb < 0)
+#endif
     for (int e0 = sp.gA + 4 * tid; e0 < sp.gB; e0 += 8 * TB) {
       const int e1 = e0 + 4 * TB;
       const bool two = e1 < sp.gB;
@@ -1785,10 +1811,12 @@ void window_rank_fill_kernel(
         tcblockOffset[gt] = (int)pos;
         tcblockRowid[gt] = w;
         // two calls, so that each store knows its address space (LDS or global)
+#ifndef F3S_PROBE_PRE_NO_TILEIDS
         if (staged)
           walk_tile_ids<W>(words, stage, pos - a0);
         else
           walk_tile_ids<W>(words, tcblocktileId, pos);
+#endif
       }
       if (staged && waveTot != 0u) {
         wave_lds_sync();
@@ -2213,7 +2241,8 @@ int launch_preprocess(const int32_t* rowPtr, const int32_t* colIdx, int N, int E
       return rc;                                                                               \
     hipLaunchKernelGGL((window_rank_fill_kernel<WW, kRankFillThreads>), dim3(nRW),            \
                        dim3(kRankFillThreads), ldsFill,                                          \
-                       stream, rowPtr, colIdx, N, E, range, chunkBytes, rowWindowOffset, hdr,  \
+                       stream, rowPtr, colIdx, N, E, range, chunkBytes, rowWindowOffset,       \
+                       sortedRowWindows, hdr,                                                  \
                        edgeToColumn, edgeToRow, tcblockRowid, tcblocktileId, tcblockOffset,    \
                        sparseAToXidx, reinterpret_cast<unsigned long long*>(bitmap));          \
     F3S_HIP_CHECK(hipGetLastError());                                                          \
