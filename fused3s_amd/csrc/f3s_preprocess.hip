@@ -798,9 +798,19 @@ __global__ __launch_bounds__(kFinBlock) void finalize_count_kernel(
     };
     // histogram of the wave's chunk: LDS atomics (the whole workgroup shares one CU's vector
     // ALUs, and a ballot per digit bit costs far more instructions than the atomic's conflicts)
+    // Counts cluster (most windows of a skewed graph share a digit), and lanes that name the same
+    // bin are served one after the other: the lanes that agree with the group's first one are
+    // counted with one ballot and added once.
     wave_lds_sync();
-    for (int i = cBegin + lane; i < cEnd; i += 64)
-      atomicAdd(&sCnt[wave][(int)(load_key(i) >> shift) & (NB - 1)], 1u);
+    for (int base = cBegin; base < cEnd; base += 64) {
+      const int i = base + lane;
+      const bool valid = i < cEnd;
+      const int dgt = (int)(load_key(i) >> shift) & (NB - 1);
+      const int d0 = __builtin_amdgcn_readfirstlane(dgt);
+      const unsigned long long same = __ballot(valid && dgt == d0);
+      if (valid && dgt != d0) atomicAdd(&sCnt[wave][dgt], 1u);
+      if (lane == 0) atomicAdd(&sCnt[wave][d0], (unsigned)__popcll(same));
+    }
     __syncthreads();
     // start of (digit = lane, wave): all smaller digits, then the same digit in earlier waves
     unsigned digitTotal = 0, before = 0;
