@@ -330,6 +330,9 @@ def run_config(name, args, dev, headline):
         "roofline": roofline,
         "traffic_recorded": recorded_traffic(name, schedule, scale_graph, natural),
     }
+    if result["traffic_recorded"] is not None:
+        # HBM-side bytes per call of the same kernels on the same workload, from the record
+        roofline["traffic"] = result["traffic_recorded"].get("bytes")
     if heads > 1:
         # the reference's way: one launch per head on contiguous per-head copies
         per_head = [tuple(x[:, h].contiguous() for x in (Q, K, V)) for h in range(heads)]
