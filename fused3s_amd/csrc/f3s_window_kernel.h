@@ -89,14 +89,50 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
 
   static_assert(!PERSIST || (!CLOCKED && !HEADS && !W8), "the persistent form is single-head");
   __shared__ int sNextPos[2];
+  __shared__ int sUnitCount;
+  __shared__ int sUnitList[NWAVES * 64];
   int pos = HEADS ? (int)(blockIdx.x / (unsigned)nHeads) : (int)blockIdx.x;
-  const int head = HEADS ? (int)(blockIdx.x - (unsigned)pos * (unsigned)nHeads) : 0;
+  int head = HEADS ? (int)(blockIdx.x - (unsigned)pos * (unsigned)nHeads) : 0;
+  // A launch that shares the windows with the wave-per-window kernel (minBlocks >= 0) covers the
+  // (position, head) units of the order's first nPositions positions with a grid of its own
+  // size: thread t of workgroup b looks at unit b + t * gridDim.x, and the workgroup computes
+  // the units it finds long, one after the other. When no window is long, which is the usual
+  // case on a graph of short windows, the launch is a thousand workgroups that read a count each
+  // and leave, instead of one workgroup per unit; in a heavy-first order the long units are the
+  // first ones and are dealt out round-robin.
+  const bool scan = !PERSIST && minBlocks >= 0;
+  int nMine = 1;
+  if (scan) {
+    if (threadIdx.x == 0) sUnitCount = 0;
+    __syncthreads();
+    const int heads = HEADS ? nHeads : 1;
+    const int64_t nUnits = (int64_t)nPositions * heads;
+    const int64_t u = (int64_t)blockIdx.x + (int64_t)threadIdx.x * (int64_t)gridDim.x;
+    if (u < nUnits) {
+      const int p = (int)(u / heads);
+      const int w = windowOrder ? windowOrder[p] : p;
+      if ((unsigned)w < (unsigned)nRW) {
+        const int t0 = rowWindowOffset[w];
+        const int t1 = rowWindowOffset[w + 1];
+        if (t0 >= 0 && (int64_t)t1 <= nTcb && t1 - t0 > minBlocks)
+          sUnitList[atomicAdd(&sUnitCount, 1)] = (int)u;
+      }
+    }
+    __syncthreads();
+    nMine = sUnitCount;
+  }
   const int pitchOut = HEADS ? ldOut : D;
   const int lane = threadIdx.x & 63;
   const int wave = pipe::uniform(threadIdx.x >> 6);
   const int g = lane >> 4;
   const int c = lane & 15;
   for (int iter = 0;; iter++) {
+  if (scan) {
+    if (iter >= nMine) break;
+    const int u = sUnitList[iter];
+    pos = HEADS ? u / nHeads : u;
+    head = HEADS ? u - pos * nHeads : 0;
+  }
   if constexpr (PERSIST) {
     if (pos >= nPositions) break;
     // position of the window after this one; read at the end of this iteration
@@ -197,9 +233,11 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
     *reinterpret_cast<float4*>(out + row * pitchOut + head * D + cv * 4) = acc;
   }
   } while (false);
-  if constexpr (!PERSIST) break;
+  if constexpr (!PERSIST) {
+    if (!scan) break;
+  }
   __syncthreads();  // the merge buffers are free again, the next position has arrived
-  pos = sNextPos[iter & 1];
+  if constexpr (PERSIST) pos = sNextPos[iter & 1];
   }
   if constexpr (CLOCKED) {
     // {first tick, last tick, CU} of this workgroup, as the reference's timed kernels record
@@ -262,9 +300,15 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
                        hl.nHeads > 0 ? hl.ldIn : D, hl.nHeads > 0 ? hl.ldOut : D,               \
                        (float*)nullptr, hl.minBlocks, (int)gw);                                 \
   }
+  // a launch next to the wave-per-window kernel looks for its units itself (see the kernel):
+  // 256 units per workgroup at most, 1024 workgroups when that is enough
+  const unsigned units = gw * (unsigned)(hl.nHeads > 0 ? hl.nHeads : 1);
+  unsigned scanGrid = (units + NWAVES * 64 - 1) / (NWAVES * 64);
+  if (scanGrid < 1024u) scanGrid = units < 1024u ? units : 1024u;
+  const bool scan = hl.minBlocks >= 0;
   bool launched = false;
   if constexpr (!WIDE) {
-    if (hl.nHeads == 0 && !cuTimer && window_cursor_requested()) {
+    if (hl.nHeads == 0 && !cuTimer && hl.minBlocks < 0 && window_cursor_requested()) {
       // F3S_WINDOW_PERSISTENT=1: as many workgroups as the GPU holds at once, windows drawn from
       // a cursor (measured slower than launch order, which therefore stays the default)
       auto kernel = f3s_fwd_kernel<ET, D, NWAVES, SOFTMAX, false, false, false, false, true>;
@@ -285,11 +329,11 @@ int launch_d(const int32_t* rwo, const int32_t* order, const int32_t* atox, cons
   }
   if (launched) {
   } else if (hl.nHeads > 0) {
-    F3S_LAUNCH(false, true, gw * (unsigned)hl.nHeads)
+    F3S_LAUNCH(false, true, scan ? scanGrid : units)
   } else if (cuTimer) {
-    F3S_LAUNCH(true, false, gw)
+    F3S_LAUNCH(true, false, scan ? scanGrid : gw)
   } else {
-    F3S_LAUNCH(false, false, gw)
+    F3S_LAUNCH(false, false, scan ? scanGrid : gw)
   }
 #undef F3S_LAUNCH
   F3S_HIP_CHECK(hipGetLastError());
