@@ -108,3 +108,54 @@ def test_split_multi_head_equals_per_head(oracle_mod, dtype):
         got = single.cpu().numpy()
         assert np.abs(got - want).max() < MAX_ABS
         assert np.abs(got - want).mean() / np.abs(want).mean() < MEAN_REL[dtype]
+
+
+def test_many_long_units_per_workgroup(oracle_mod):
+    """More long (window, head) units than the long-window launch has workgroups (1024): its
+    workgroups find several units each and compute them one after the other. 40 000 rows, one
+    edge per row on average, 310 windows whose rows name 40 columns each; eight heads."""
+    from fused3s_amd import capi
+    print("case short_windows many long units", flush=True)
+    N, heads, d = 40000, 8, 32
+    rng = np.random.default_rng(11)
+    deg = rng.poisson(1.0, N)
+    for w in range(0, N // 16, 8)[:310]:
+        deg[16 * w:16 * w + 16] = 40
+    rowPtr = np.zeros(N + 1, np.int32)
+    rowPtr[1:] = np.cumsum(deg)
+    colIdx = np.concatenate([np.sort(rng.choice(N, size=k, replace=False)) for k in deg]
+                            ).astype(np.int32)
+    pre = oracle_mod.preprocess(rowPtr, colIdx, N)
+    counts = np.diff(pre["rowWindowOffset"])
+    nRW = len(counts)
+    assert nRW >= 1024 and counts.sum() < 16 * nRW        # the split is taken
+    assert (counts > 32).sum() * heads > 2 * 1024          # two long units per workgroup and more
+    dev = "cuda"
+    rwo = torch.as_tensor(pre["rowWindowOffset"].astype(np.int32)).to(dev)
+    atox = torch.as_tensor(pre["sparseAToXidx"].astype(np.int32)).to(dev)
+    bm = torch.as_tensor(pre["tcbBitMap"].view(np.int64)).to(dev).view(torch.uint64)
+    heavy_first = torch.as_tensor(pre["sortedRowWindows"].astype(np.int32)).to(dev)
+    g = torch.Generator().manual_seed(3)
+    shuffled = heavy_first[torch.randperm(nRW, generator=g).to(dev)].contiguous()
+    Q, K, V = [(torch.randn((N, heads, d), generator=g) * d ** -0.25).to(torch.bfloat16).to(dev)
+               for _ in range(3)]
+    scale = float(np.sqrt(d))
+    want = [oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"],
+                                     pre["tcbBitMap"], N, bits(Q[:, h]), bits(K[:, h]),
+                                     bits(V[:, h]), scale, dtype=1) for h in range(heads)]
+    for name, order in (("heavy_first", heavy_first), ("shuffled", shuffled)):
+        out = torch.full((N, heads * d), float("nan"), dtype=torch.float32, device=dev)
+        capi.attention_heads(rwo, order, atox, bm, N, Q, K, V, scale, out=out)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all(), name  # every row written by exactly one of the kernels
+        for h in range(heads):
+            gh = got[:, h * d:(h + 1) * d]
+            assert np.abs(gh - want[h]).max() < MAX_ABS, (name, h)
+            assert np.abs(gh - want[h]).mean() / np.abs(want[h]).mean() < MEAN_REL[torch.bfloat16]
+    # single head through the same launch shape
+    q1, k1, v1 = (x[:, 0].contiguous() for x in (Q, K, V))
+    out1 = torch.full((N, d), float("nan"), dtype=torch.float32, device=dev)
+    capi.attention(rwo, heavy_first, atox, bm, N, q1, k1, v1, scale, out=out1)
+    torch.cuda.synchronize()
+    assert np.abs(out1.cpu().numpy() - want[0]).max() < MAX_ABS
