@@ -58,7 +58,7 @@ __device__ __forceinline__ pipe::Problem<ET> make_problem(const int32_t* sparseA
                                                           const uint8_t* bitmapBytes, const ET* Q,
                                                           const ET* K, const ET* V, int N,
                                                           float scaleLog2, int ldIn,
-                                                          int64_t nTcb) {
+                                                          int64_t nTcb, int ldQ = 0) {
   pipe::Problem<ET> pb;
   pb.sparseAToXidx = sparseAToXidx;
   pb.bitmapBytes = bitmapBytes;
@@ -68,6 +68,7 @@ __device__ __forceinline__ pipe::Problem<ET> make_problem(const int32_t* sparseA
   pb.N = N;
   pb.scaleLog2 = scaleLog2;
   pb.pitchIn = HEADS ? ldIn : D;
+  pb.pitchQ = (HEADS && ldQ > 0) ? ldQ : pb.pitchIn;  // Q may lie apart from K / V
   pb.nTcb = nTcb;
   pb.sddmm = nullptr;
   return pb;
@@ -117,7 +118,7 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
                     int64_t nTcb, const ET* __restrict__ Q, const ET* __restrict__ K,
                     const ET* __restrict__ V, float scaleLog2, float* __restrict__ partial,
                     float* __restrict__ out, int nHeads, int ldIn, int ldOut, int maxBlocks,
-                    int longPrefix) {
+                    int longPrefix, int ldQ) {
   typedef pipe::PairPipeline<ET, D, SOFTMAX, HEADS, false> Pipe;
   constexpr int T = D / 16;
   extern __shared__ __align__(1024) unsigned char smem[];
@@ -158,7 +159,7 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
   if (t0 < 0 || (int64_t)t1 > nTcb) return;
 
   const pipe::Problem<ET> pb = make_problem<ET, D, HEADS>(sparseAToXidx, bitmapBytes, Q, K, V, N,
-                                                          scaleLog2, ldIn, nTcb);
+                                                          scaleLog2, ldIn, nTcb, ldQ);
   const unsigned ringAddr =
       (unsigned)(uintptr_t)(F3S_LDS unsigned char*)smem + (unsigned)wave * pipe::Geo<D>::WAVE_BYTES;
   Pipe pp;
@@ -481,17 +482,52 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 struct SlicedLayout {
   int P, S;
   size_t tickets, sliceStart, partial, total;
+  size_t padded;  // 0, or where the copies of K and V with 256-byte rows start (single head, d = 64)
 };
+// Rows of 128 bytes gathered from addresses that are multiples of 256 are served faster than rows
+// from the odd 128-byte lines in between (233k-node graph, d = 64: 1.42 ms with every row on an
+// even line, 1.55 ms with every row on an odd line, 1.48 ms for contiguous rows, which alternate;
+// the L2 hit and miss counts are the same in all three). The single-head call at d = 64 therefore
+// gathers from copies of K and V with a row pitch of 256 bytes, made at the start of the call.
+constexpr int kPaddedRowBytes = 256;
+// nHeads = 0: the single-head layout
 SlicedLayout sliced_layout(int N, int d, int nHeads) {
+  const int heads = nHeads > 0 ? nHeads : 1;
   SlicedLayout L;
-  L.P = choose_phases(N, d * nHeads);
+  L.P = choose_phases(N, d * heads);
   L.S = L.P * kXcds;
   const size_t nRW = (size_t)(N + kWinRows - 1) / kWinRows;
   L.tickets = 256;
   L.sliceStart = L.tickets + 256;
   L.partial = L.sliceStart + align256(nRW * (L.S + 1) * sizeof(int32_t));
-  L.total = L.partial + nRW * nHeads * L.S * (size_t)(d / 4 + 2) * 64 * sizeof(float);
+  L.total = align256(L.partial + nRW * heads * L.S * (size_t)(d / 4 + 2) * 64 * sizeof(float));
+  L.padded = 0;
+  if (nHeads == 0 && d == 64) {
+    L.padded = L.total;
+    L.total += 2 * (size_t)N * kPaddedRowBytes;
+  }
   return L;
+}
+
+// K and V rows of 128 bytes copied to a pitch of 256 bytes (one thread per 16 bytes of each)
+typedef int pad_chunk __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void pad_rows_kernel(const pad_chunk* __restrict__ K,
+                                                       const pad_chunk* __restrict__ V,
+                                                       int64_t chunks, pad_chunk* __restrict__ Kp,
+                                                       pad_chunk* __restrict__ Vp) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= chunks) return;
+  const int64_t row = i >> 3;
+  const int c = (int)(i & 7);
+  const pad_chunk k = __builtin_nontemporal_load(K + i);  // read once, by nobody else
+  const pad_chunk v = __builtin_nontemporal_load(V + i);
+  Kp[row * (kPaddedRowBytes / 16) + c] = k;
+  Vp[row * (kPaddedRowBytes / 16) + c] = v;
+}
+
+bool padded_rows_requested() {
+  const char* e = getenv("F3S_PAD_ROWS");  // read per call; 0 switches the copies off
+  return !(e && e[0] == '0');
 }
 
 // workgroups of NW waves the GPU holds at once (LDS rings, waves per SIMD), a multiple of 8
@@ -528,7 +564,7 @@ int launch_sliced_units(const int32_t* rwo, const int32_t* order, const int32_t*
                         const uint8_t* bm, int N, int nRW, const ET* Q, const ET* K, const ET* V,
                         float scaleLog2, float* out, int32_t* tickets, int32_t* sliceStart,
                         float* partial, const SlicedLayout& L, int heads, int ldIn, int ldOut,
-                        int64_t nTcb, hipStream_t stream) {
+                        int64_t nTcb, hipStream_t stream, int ldQ = 0) {
   constexpr size_t lds = (size_t)kUnitWaves * pipe::Geo<D>::WAVE_BYTES;
   if (resident_requested()) {
     auto kernel = f3s_fwd_resident_kernel<ET, D, SOFTMAX, HEADS, kUnitWaves>;
@@ -547,7 +583,7 @@ int launch_sliced_units(const int32_t* rwo, const int32_t* order, const int32_t*
       return fail(-2, "f3s_attention: too many (window, slice, head) units for one launch");
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kUnitWaves * 64), lds, stream, order, rwo,
                        atox, bm, sliceStart, L.S, (int)nGroups, N, nRW, nTcb, Q, K, V, scaleLog2,
-                       partial, out, heads, ldIn, ldOut, 0, 0);
+                       partial, out, heads, ldIn, ldOut, 0, 0, ldQ);
   }
   F3S_HIP_CHECK(hipGetLastError());
   return 0;
@@ -576,14 +612,31 @@ int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* ato
   const auto* q = static_cast<const ET*>(Q);
   const auto* k = static_cast<const ET*>(K);
   const auto* v = static_cast<const ET*>(V);
-  const int rc =
-      nHeads > 0
-          ? launch_sliced_units<ET, D, SOFTMAX, true>(rwo, order, atox, bm, N, nRW, q, k, v,
-                                                      scaleLog2, out, tickets, sliceStart, partial,
-                                                      L, heads, ldIn, ldOut, nTcb, stream)
-          : launch_sliced_units<ET, D, SOFTMAX, false>(rwo, order, atox, bm, N, nRW, q, k, v,
-                                                       scaleLog2, out, tickets, sliceStart, partial,
-                                                       L, 1, D, D, nTcb, stream);
+  int rc;
+  if (nHeads > 0) {
+    rc = launch_sliced_units<ET, D, SOFTMAX, true>(rwo, order, atox, bm, N, nRW, q, k, v,
+                                                   scaleLog2, out, tickets, sliceStart, partial, L,
+                                                   heads, ldIn, ldOut, nTcb, stream);
+  } else if (L.padded != 0 && padded_rows_requested() && !resident_requested() &&
+             !gather_needs_wide_offsets(N, kPaddedRowBytes, true)) {
+    // copies of K and V with 256-byte rows, gathered through the pitched (multi-head) form of the
+    // unit kernel with one head; Q stays where it is
+    auto* kp = reinterpret_cast<ET*>(ws + L.padded);
+    auto* vp = kp + (size_t)N * (kPaddedRowBytes / sizeof(ET));
+    const int64_t chunks = (int64_t)N * (D * (int)sizeof(ET) / 16);
+    hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                       stream, reinterpret_cast<const pad_chunk*>(k),
+                       reinterpret_cast<const pad_chunk*>(v), chunks,
+                       reinterpret_cast<pad_chunk*>(kp), reinterpret_cast<pad_chunk*>(vp));
+    F3S_HIP_CHECK(hipGetLastError());
+    rc = launch_sliced_units<ET, D, SOFTMAX, true>(
+        rwo, order, atox, bm, N, nRW, q, kp, vp, scaleLog2, out, tickets, sliceStart, partial, L, 1,
+        kPaddedRowBytes / (int)sizeof(ET), D, nTcb, stream, D);
+  } else {
+    rc = launch_sliced_units<ET, D, SOFTMAX, false>(rwo, order, atox, bm, N, nRW, q, k, v,
+                                                    scaleLog2, out, tickets, sliceStart, partial,
+                                                    L, 1, D, D, nTcb, stream);
+  }
   if (rc != 0) return rc;
   const int64_t merges = (int64_t)nRW * heads;
   hipLaunchKernelGGL((f3s_merge_slices_kernel<D, SOFTMAX>), dim3((unsigned)((merges + 3) / 4)),
@@ -596,7 +649,7 @@ int launch_sliced_d(const int32_t* rwo, const int32_t* order, const int32_t* ato
 }  // namespace
 
 size_t attention_sliced_workspace_bytes(int N, int d, int nHeads) {
-  return sliced_layout(N, d, nHeads > 0 ? nHeads : 1).total;
+  return sliced_layout(N, d, nHeads).total;
 }
 
 // mode 0 / 2: an attention call (2: on a prepared workspace); mode 1: f3s_attention_prepare
@@ -609,7 +662,7 @@ int launch_attention_sliced(const int32_t* rowWindowOffset, const int32_t* windo
                             int mode, hipStream_t stream) {
   if (!head_dim_supported(d))
     return fail(-2, "f3s_attention: head dim %d unsupported (a multiple of 32 up to 256)", d);
-  const SlicedLayout L = sliced_layout(N, d, nHeads > 0 ? nHeads : 1);
+  const SlicedLayout L = sliced_layout(N, d, nHeads);
   if (wsBytes < L.total)
     return fail(-2, "f3s_attention: workspace %zu B < required %zu B", wsBytes, L.total);
   char* ws = static_cast<char*>(workspace);
@@ -658,12 +711,12 @@ int launch_short_d(const int32_t* rwo, const int32_t* order, const int32_t* atox
     if (int rc = allow_lds(f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, true>, lds)) return rc;
     hipLaunchKernelGGL((f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, true>), grid, block, lds,
                        stream, order, rwo, atox, bm, nullptr, 0, 0, N, (int)nRW, nTcb, q, k, v,
-                       scaleLog2, nullptr, out, nHeads, ldIn, ldOut, maxBlocks, longPrefix);
+                       scaleLog2, nullptr, out, nHeads, ldIn, ldOut, maxBlocks, longPrefix, 0);
   } else {
     if (int rc = allow_lds(f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, false>, lds)) return rc;
     hipLaunchKernelGGL((f3s_fwd_unit_kernel<ET, D, SOFTMAX, false, false>), grid, block, lds,
                        stream, order, rwo, atox, bm, nullptr, 0, 0, N, (int)nRW, nTcb, q, k, v,
-                       scaleLog2, nullptr, out, 1, D, D, maxBlocks, longPrefix);
+                       scaleLog2, nullptr, out, 1, D, D, maxBlocks, longPrefix, 0);
   }
   F3S_HIP_CHECK(hipGetLastError());
   return 0;

@@ -264,7 +264,8 @@ struct Problem {
   const ET* __restrict__ V;
   int N;
   float scaleLog2;   // log2(e) / scalingFactor (1.0 without softmax)
-  int pitchIn;       // row pitch of Q/K/V in elements (D for the single-head layout)
+  int pitchIn;       // row pitch of K/V in elements (D for the single-head layout)
+  int pitchQ;        // row pitch of Q in elements
   int64_t nTcb;      // TC blocks in sparseAToXidx / bitmapBytes (bounds of the metadata loads)
   float* __restrict__ sddmm;  // 16x8 structure only: masked unscaled scores, or null
 };
@@ -321,7 +322,7 @@ struct PairPipeline {
       const int64_t qrow = (int64_t)w * 16 + c;
       if (qrow < pb.N) {
         const half8* qp =
-            reinterpret_cast<const half8*>(pb.Q + qrow * pb.pitchIn + (HEADS ? head * D : 0)) + g;
+            reinterpret_cast<const half8*>(pb.Q + qrow * pb.pitchQ + (HEADS ? head * D : 0)) + g;
 #pragma unroll
         for (int i = 0; i < KS; i++) qf[i] = qp[4 * i];
       } else {

@@ -161,6 +161,7 @@ __attribute__((amdgpu_waves_per_eu(waves_per_simd(D), waves_per_simd(D)))) void 
   pb.N = N;
   pb.scaleLog2 = scaleLog2;
   pb.pitchIn = HEADS ? ldIn : D;
+  pb.pitchQ = pb.pitchIn;
   pb.nTcb = nTcb;
   pb.sddmm = sddmm;
   const unsigned ringAddr =

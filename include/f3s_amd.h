@@ -189,8 +189,11 @@ int f3s_attention_fwd(const int32_t* rowWindowOffset, const int32_t* windowOrder
 /*
  * Bytes of device scratch f3s_attention_fwd / f3s_attention_fwd_heads can use for a graph of N
  * nodes at head dimension d (a header, the slice boundaries of every window, plus one partial
- * (m, l, O) per window, head and slice: about 4.6 KB * ceil(N/16) * slices at d = 64). The reference's launchers (src/F3S_kernel.cu:581-671) need no scratch;
- * passing workspace = NULL keeps that behaviour.
+ * (m, l, O) per window, head and slice: about 4.6 KB * ceil(N/16) * slices at d = 64; for the
+ * single-head call at d = 64 also 512 * N bytes for copies of K and V with 256-byte rows, which
+ * the call makes itself and gathers from instead: rows that start on even 128-byte lines are
+ * served faster than rows on the odd lines in between). The reference's launchers
+ * (src/F3S_kernel.cu:581-671) need no scratch; passing workspace = NULL keeps that behaviour.
  */
 size_t f3s_attention_workspace_bytes(int N, int d);
 size_t f3s_attention_heads_workspace_bytes(int N, int nHeads, int d);

@@ -200,6 +200,41 @@ def test_schedule_switches_are_read_per_call(oracle_mod, long_window_graph, monk
     assert np.array_equal(outs[0], outs[2])
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_padded_row_copies_change_nothing(oracle_mod, long_window_graph, monkeypatch, dtype):
+    """At d = 64 the single-head column-sliced call gathers from copies of K and V with 256-byte
+    rows that it makes in its workspace (F3S_PAD_ROWS=0 switches them off): same arithmetic on the
+    same values, so the results are bit-identical, with and without a prepared workspace, and meet
+    the oracle. K and V are changed between calls: the copies are made per call."""
+    from fused3s_amd import capi
+    print("case padded rows %s" % dtype, flush=True)
+    N, _, _, pre = long_window_graph
+    rwo, order, atox, bm = to_dev(pre)
+    g = torch.Generator().manual_seed(64)
+    Q, K, V = [torch.randn((N, 64), generator=g).to(dtype).cuda() for _ in range(3)]
+    code = 0 if dtype == torch.float16 else 1
+    L = capi.lib()
+    assert L.f3s_attention_workspace_bytes(N, 64) >= 2 * N * 256  # room for the copies
+    ws = capi.attention_workspace(N, 64, "cuda")
+    outs = {}
+    for flag in ("1", "0"):
+        monkeypatch.setenv("F3S_PAD_ROWS", flag)
+        outs[flag] = capi.attention(rwo, order, atox, bm, N, Q, K, V, 8.0, workspace=ws).clone()
+    assert torch.equal(outs["1"], outs["0"])
+    want = oracle_mod.attention_ref(pre["rowWindowOffset"], pre["sparseAToXidx"], pre["tcbBitMap"],
+                                    N, bits(Q), bits(K), bits(V), 8.0, dtype=code)
+    got = outs["1"].cpu().numpy()
+    assert np.abs(got - want).max() < MAX_ABS and mean_rel(got, want) < MEAN_REL
+    monkeypatch.setenv("F3S_PAD_ROWS", "1")
+    capi.attention_prepare(rwo, atox, N, 64, ws)
+    K2, V2 = V.clone(), K.clone()  # other values in the same call sequence
+    a = capi.attention(rwo, order, atox, bm, N, Q, K2, V2, 8.0, workspace=ws, prepared=True).clone()
+    monkeypatch.setenv("F3S_PAD_ROWS", "0")
+    b = capi.attention(rwo, order, atox, bm, N, Q, K2, V2, 8.0, workspace=ws, prepared=True)
+    assert torch.equal(a, b) and not torch.equal(a, outs["1"])
+
+
 def test_wide_offset_rule():
     """Host side of the 64-bit row offsets: which problems take them (no GPU needed)."""
     from fused3s_amd import capi
