@@ -132,6 +132,15 @@ preprocess_gpu(torch::Tensor edgeList, torch::Tensor nodePointer, int num_nodes,
     tcblockOffset = tcblockOffset.narrow(0, 0, nTcb + 1);
     sparseAToXidx = sparseAToXidx.narrow(0, 0, nTcb * blockSize_w);
     tcbBitMap = tcbBitMap.narrow(0, 0, nTcb * bmWords);
+    if (nTcb * 2 < cap) {
+      // rows of a window that share columns: far fewer blocks than the bound. The views would keep
+      // the whole allocation alive for as long as the caller keeps the structure, so it gets
+      // exact-size copies instead (at most half of what was allocated is copied).
+      tcblockRowid = tcblockRowid.clone();
+      tcblockOffset = tcblockOffset.clone();
+      sparseAToXidx = sparseAToXidx.clone();
+      tcbBitMap = tcbBitMap.clone();
+    }
   }
   if (verbose()) {
     TORCH_CHECK(hipStreamSynchronize(at::hip::getCurrentHIPStream().stream()) == hipSuccess);

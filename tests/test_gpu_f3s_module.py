@@ -120,6 +120,11 @@ def test_preprocess_gpu_both_allocation_styles(oracle_mod, monkeypatch, W):
     graphs = [long_window_graph(rng, 2000, 180, messy_every=60, empty_every=13)]
     rp, ci, _, _, _ = reference_style_inputs(1000, 32)
     graphs.append((rp, ci))
+    # the sixteen rows of a window name the same 64 columns: a sixteenth of the blocks that the
+    # bound allows, so the default style hands out exact-size copies, not views
+    shared = np.concatenate([np.tile(np.sort(rng.choice(1600, 64, replace=False)), 16)
+                             for _ in range(100)]).astype(np.int32)
+    graphs.append((np.arange(0, 1600 * 64 + 1, 64, dtype=np.int32), shared))
     for rowPtr, colIdx in graphs:
         N = len(rowPtr) - 1
         print("case module allocation styles N=%d E=%d W=%d" % (N, len(colIdx), W), flush=True)
@@ -133,6 +138,10 @@ def test_preprocess_gpu_both_allocation_styles(oracle_mod, monkeypatch, W):
             assert rowid.numel() == count and toff.numel() == count + 1
             assert atox.numel() == count * W and bm.numel() == count * 16 * W // 64
             assert all(t.is_contiguous() for t in (rowid, toff, atox, bm, tile))
+            bound = (len(colIdx) + W - 1) // W + (N + 15) // 16
+            if count * 2 < bound:  # no tensor keeps the bounded allocation alive
+                assert atox.untyped_storage().nbytes() == atox.numel() * 4
+                assert bm.untyped_storage().nbytes() == bm.numel() * 8
             got = dict(rowWindowOffset=rwo, sortedRowWindows=order, tcblockRowid=rowid,
                        tcblocktileId=tile, tcblockOffset=toff, sparseAToXidx=atox,
                        blockCount=count,
