@@ -231,7 +231,42 @@ def run_config(name, args, dev, headline):
     log("attention schedule: %s" % ("column-sliced (%.0f MB workspace)" % (workspace.numel() / 1e6)
                                     if workspace is not None else "workgroup per window"))
 
-    if heads == 1:
+    layout = getattr(args, "kv_layout", "") if headline else ""
+    if heads == 1 and layout:
+        # experiment: K and V rows placed differently in memory, through the multi-head entry
+        # with one head (which takes any row pitch); the values are the same
+        def placed(t, pitch_bytes, offset_bytes=0, store=None):
+            pe, oe = pitch_bytes // t.element_size(), offset_bytes // t.element_size()
+            if store is None:
+                store = torch.zeros((N, pe), dtype=t.dtype, device=dev)
+            store[:, oe:oe + d] = t
+            return store[:, oe:oe + d].unflatten(1, (1, d)), store
+        row = d * Q.element_size()
+        if layout == "interleaved":  # one array of 2-row records: K in the first half, V behind it
+            pitch = 2 * row
+            Kh, kv = placed(K, pitch)
+            Vh, _ = placed(V, pitch, row, kv)
+        elif layout.startswith("odd"):  # rows at pitch P, each one row beyond the pitch boundary
+            pitch = int(layout[3:])
+            Kh, _ = placed(K, pitch, row)
+            Vh, _ = placed(V, pitch, row)
+        else:  # "pitch<bytes>"
+            pitch = int(layout[5:])
+            Kh, _ = placed(K, pitch)
+            Vh, _ = placed(V, pitch)
+        Qh, _ = placed(Q, pitch)  # the entry takes one pitch for Q, K and V
+        workspace = capi.attention_workspace(N, d, dev, nTCB=nTCB, dtype=tdtype, heads=1)
+        if workspace is not None:
+            capi.attention_prepare(pre["rowWindowOffset"], pre["sparseAToXidx"], N, d, workspace,
+                                   heads=1)
+        log("K / V layout: %s (multi-head entry, one head)" % layout)
+
+        def step(v=V, o=out):
+            vh = Vh if v is V else placed(v, pitch)[0]
+            capi.attention_heads(pre["rowWindowOffset"], order, pre["sparseAToXidx"],
+                                 pre["tcbBitMap"], N, Qh, Kh, vh, scale, True, out=o,
+                                 workspace=workspace, prepared=workspace is not None)
+    elif heads == 1:
         def step(v=V, o=out):
             capi.attention(pre["rowWindowOffset"], order, pre["sparseAToXidx"], pre["tcbBitMap"],
                            N, Q, K, v, scale, True, out=o, workspace=workspace,
@@ -384,6 +419,10 @@ def main():
     ap.add_argument("--two-phase-preprocess", action="store_true",
                     help="preprocess with f3s_preprocess_count + f3s_preprocess_fill instead of "
                          "the one call f3s_preprocess")
+    ap.add_argument("--kv-layout", default="",
+                    help="experiment on a single-head configuration: K / V rows at pitch<bytes>, "
+                         "odd<bytes> (one row beyond every pitch boundary) or interleaved, through "
+                         "the multi-head entry with one head")
     ap.add_argument("--preprocess-only", action="store_true",
                     help="time the preprocessing of --config and stop (no attention call)")
     ap.add_argument("--cpu-budget", type=float, default=12.0)
