@@ -46,6 +46,9 @@ PROBES = {
     "no_compute": ["-DF3S_PROBE_NO_COMPUTE"],
     # LDS reads and arithmetic on whatever the first two steps left in the ring, no gather
     "no_gather": ["-DF3S_PROBE_NO_GATHER"],
+    # column-sliced schedule: the four waves of a workgroup all compute the workgroup's first
+    # unit, at the same time (what the L1 makes of rows that several waves ask for together)
+    "same_unit": ["-DF3S_PROBE_SAME_UNIT"],
     # Preprocessing (window_rank_fill_kernel) with one part left out. Their block arrays are
     # incomplete: time them with `python bench.py --preprocess-only` and never hand what they
     # produce to an attention call (bench.py refuses to).

@@ -133,7 +133,12 @@ f3s_fwd_unit_kernel(const int32_t* __restrict__ windowOrder,
     const int xcd = blockIdx.x % kXcds;
     const int j = blockIdx.x / kXcds;
     const int phase = j / nGroups;
+#ifdef F3S_PROBE_SAME_UNIT
+    // probe: the four waves of a workgroup all compute its first unit, at the same time
+    const int64_t u = (int64_t)(j - phase * nGroups) * (int)(blockDim.x >> 6);
+#else
     const int64_t u = (int64_t)(j - phase * nGroups) * (int)(blockDim.x >> 6) + wave;
+#endif
     const int pos = HEADS ? (int)(u / nHeads) : (int)u;
     head = HEADS ? (int)(u - (int64_t)pos * nHeads) : 0;
     if (pos >= nRW) return;
